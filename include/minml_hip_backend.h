@@ -1,0 +1,155 @@
+/*
+ * minml_hip_backend.h — C-ABI of the MI355X (gfx950) HIP backend for minml's convolution / GEMM inference path.
+ *
+ * Every entry point mirrors, argument for argument, the device-backend entry point that minml's core dispatcher
+ * (reference: src/core/math.cpp, src/core/ml_memory.cpp, src/core/Context.cpp, src/core/Event.cpp) calls in its
+ * DeviceType::CUDA branch, declared in the reference at include/minml/backend/cuda_backend.h. The library exports
+ * each function twice: under the hip_* name declared here and under the cuda_* name of the reference, so that the
+ * unmodified dispatcher links against it in place of src/backend/cuda_dummy_backend.cpp.
+ *
+ * Conventions (same as the reference backends):
+ *   - descriptors are passed by value; all tensors are dense, row-major, NHWC for images;
+ *   - an absent optional tensor is signalled by data == NULL (reference: include/minml/backend/backend_utils.hpp:138-141);
+ *   - every call is asynchronous on the context's stream; hip_synchronize_with_context is the only barrier;
+ *   - failures are C++ exceptions crossing the C boundary (std::runtime_error / std::logic_error), never return codes
+ *     (reference: src/backend/cuda_dummy_backend.cpp:25-27, src/backend/cpu/winograd/winograd_runtime.cpp:516).
+ */
+#ifndef MINML_HIP_BACKEND_H_
+#define MINML_HIP_BACKEND_H_
+
+#include <stddef.h>
+#include <stdbool.h>
+
+#ifdef __cplusplus
+extern "C"
+{
+#endif
+
+/* ---- descriptor types: binary-compatible with reference include/minml/backend/backend_types.h:28-73 ---- */
+#ifndef MINML_BACKEND_BACKEND_TYPES_H_
+	typedef struct
+	{
+		int rank;
+		int dim[6];
+	} mlShape_t;
+
+	typedef struct
+	{
+		float scale;
+		float shift;
+	} mlQuantizationData_t;
+
+	typedef enum
+	{
+		DTYPE_UNKNOWN, DTYPE_FLOAT8, DTYPE_FLOAT16, DTYPE_FLOAT32, DTYPE_FLOAT64, DTYPE_UINT8, DTYPE_INT8, DTYPE_INT16, DTYPE_INT32
+	} mlDataType_t;
+
+	typedef enum
+	{
+		ACTIVATION_LINEAR, ACTIVATION_SIGMOID, ACTIVATION_TANH, ACTIVATION_RELU, ACTIVATION_LEAKY_RELU, ACTIVATION_EXP
+	} mlActivationType_t;
+
+	typedef struct
+	{
+		void *data;
+		mlDataType_t dtype;
+		int rank;
+		int dim[6];
+	} mlTensor_t;
+
+	typedef void *mlContext_t;
+	typedef void *mlEvent_t;
+#endif
+
+	/* ---- device identity (reference: cuda_backend.h:49-57, src/backend/cuda/cuda_properties.cpp) ---- */
+	int hip_get_number_of_devices(void);
+	int hip_get_memory(int index); /* in MB */
+	bool hip_supports_type(int index, mlDataType_t dtype); /* FLOAT16, FLOAT32, INT32, INT8 (cuda_properties.cpp:222-244) */
+	const char* hip_get_device_info(int index);
+	const char* hip_get_device_features(int index);
+	void hip_enable_tf32(mlContext_t context, bool b); /* accepted and ignored: fp32 GEMMs run in full fp32 */
+
+	/* ---- context = one stream (reference: cuda_backend.h:59-63, src/backend/cuda/cuda_context.cpp) ---- */
+	mlContext_t hip_create_context(int device_index);
+	void hip_synchronize_with_context(mlContext_t context);
+	bool hip_is_context_ready(mlContext_t context);
+	void hip_destroy_context(mlContext_t context);
+
+	/* ---- events (reference: cuda_backend.h:65-70, src/backend/cuda/cuda_event.cpp) ---- */
+	mlEvent_t hip_create_event(mlContext_t context); /* records on the context's stream */
+	double hip_get_time_between_events(mlEvent_t start, mlEvent_t end); /* seconds */
+	void hip_wait_for_event(mlEvent_t event);
+	bool hip_is_event_ready(mlEvent_t event);
+	void hip_destroy_event(mlEvent_t event);
+
+	/* ---- memory (reference: cuda_backend.h:72-83, src/backend/cuda/cuda_memory.cu:133-276); context == NULL => synchronous ---- */
+	void* hip_malloc(int device_index, size_t count);
+	void hip_page_lock(void *ptr, size_t count); /* no-op: registering existing host memory is not available on the target hosts */
+	void hip_page_unlock(void *ptr);
+	void hip_free(void *ptr);
+	void* hip_create_view(void *src, size_t offset, size_t count); /* src + offset, non-owning */
+	void hip_destroy_view(void *ptr);
+	void hip_memset(mlContext_t context, void *dst, size_t dst_offset, size_t dst_count, const void *src, size_t src_count); /* pattern of 0,1,2,4,8 bytes */
+	void hip_memcpy_within_device(mlContext_t context, void *dst, size_t dst_offset, const void *src, size_t src_offset, size_t count);
+	void hip_memcpy_from_host(mlContext_t context, void *dst, size_t dst_offset, const void *src, size_t count);
+	void hip_memcpy_to_host(mlContext_t context, void *dst, const void *src, size_t src_offset, size_t count);
+
+	/* ---- step before the path (reference: cuda_backend.h:85-88, src/backend/cpu/dispatcher.cpp:112-188) ---- */
+	void hip_unpack_input(mlContext_t context, mlShape_t shape, mlDataType_t dst_dtype, void *dst, const void *src);
+	void hip_convert_type(mlContext_t context, void *dst, mlDataType_t dst_dtype, const void *src, mlDataType_t src_dtype, int elements);
+
+	/* ---- Winograd F(4x4,3x3) transforms (reference: cuda_backend.h:96-100; arithmetic follows the CPU backend,
+	 *      src/backend/cpu/winograd/winograd_runtime.cpp:47-232,519-536). The kernel size is derived from
+	 *      matrices.dim[0] = (tile + k - 1)^2; any (tile, kernel, dtype) other than (4, 3, fp16|fp32) throws
+	 *      std::runtime_error("No suitable Winograd transform runtime"). ---- */
+	void hip_winograd_weight_transform(mlContext_t context, int tile_size, const mlTensor_t w, mlTensor_t matrices, bool invert);
+	void hip_winograd_input_transform(mlContext_t context, int tile_size, const mlTensor_t x, mlTensor_t matrices);
+	void hip_winograd_output_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
+			mlTensor_t y, mlActivationType_t act);
+
+	/* ---- GEMMs (reference: cuda_backend.h:147-154; semantics of src/backend/cpu/gemm/gemm.cpp:34-83).
+	 *      C.dtype == INT32 selects the int8 x int8 -> int32 product (src/backend/cuda/gemms.cpp:119-130). ---- */
+	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C);
+	void hip_gemm_batched_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C);
+	void hip_gemm(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
+			const void *B, char opA, char opB, float alpha, float beta);
+	void hip_gemm_batched(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
+			const void *B, char opA, char opB, float alpha, float beta);
+	/* D = act(alpha * op_A(A) * op_B(B) + bias + beta * C)  (reference: cuda_backend.h:160-162, src/backend/cpu/gemm/gemm.cpp:66-83) */
+	void hip_gemm_ex(mlContext_t context, mlDataType_t dtype, mlShape_t shape_D, void *D, float alpha, char opA, mlShape_t shape_A, const void *A,
+			char opB, mlShape_t shape_B, const void *B, float beta, mlShape_t shape_C, const void *C, const void *bias, mlActivationType_t act);
+
+	/* ---- fused convolution y = act(conv(x, w) + bias + add), stride 1, pad (k-1)/2, weights [Cout,k,k,Cin]
+	 *      (reference: cuda_backend.h:103-106, src/core/math.cpp:399-416; oracle = explicit_gemm_forward,
+	 *      src/core/math.cpp:1595-1626). dtype INT8 is not part of this entry point (see hip_quantized_conv_forward). ---- */
+	void hip_convolution_implicit_gemm_forward(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, mlShape_t weights_shape,
+			const void *input, const void *weights, void *output, const void *bias, const void *add, mlActivationType_t act);
+	void hip_im2row(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, void *output, const void *input, int kernel_size, bool invert,
+			const void *padding); /* reference: cuda_backend.h:326-327; `padding` = pointer to one host element or NULL for zeros */
+
+	/* ---- int8 epilogue (reference: cuda_backend.h:323-325; arithmetic of the CPU path, src/layers/Conv2D.cpp:284-306) ---- */
+	void hip_quantized_scale_shift_act(mlContext_t context, mlDataType_t dtype, mlShape_t shape, void *output, mlQuantizationData_t output_qd,
+			const void *input, const void *scales, const void *bias, mlActivationType_t act, const void *ext, mlQuantizationData_t ext_qd);
+
+	/* ---- non-fused fallbacks (reference: cuda_backend.h:172-173,222-223,296-297) ---- */
+	void hip_add_bias_act(mlContext_t context, float alpha, const mlTensor_t x, const mlTensor_t b, float beta, mlTensor_t y, mlActivationType_t act);
+	void hip_activation_forward(mlContext_t context, float alpha, const mlTensor_t x, float beta, mlTensor_t y, mlActivationType_t act);
+	void hip_add_tensors(mlContext_t context, float alpha1, const mlTensor_t x1, float alpha2, const mlTensor_t x2, float alpha3, const mlTensor_t x3,
+			float beta, mlTensor_t y);
+	void hip_scale_tensor(mlContext_t context, float alpha, mlTensor_t x); /* x *= alpha (reference: cuda_backend.h:295) */
+
+	/* ---- additions with no counterpart in the reference ABI ----
+	 * hip_quantized_conv_forward: the whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 (int8 implicit GEMM with
+	 * zero-point padding, int32 accumulation, per-channel scale + bias, optional int8 residual, activation, requantisation)
+	 * in one launch, so that neither the im2row matrix nor the int32 accumulators touch HBM. output dtype INT8 or FLOAT32. */
+	void hip_quantized_conv_forward(mlContext_t context, mlShape_t input_shape, mlShape_t weights_shape, const void *input,
+			mlQuantizationData_t input_qd, const void *weights, const void *scales, const void *bias, mlDataType_t output_dtype, void *output,
+			mlQuantizationData_t output_qd, const void *ext, mlQuantizationData_t ext_qd, mlActivationType_t act);
+	/* hip_get_stream: the hipStream_t of a context, for callers that time or capture work on it. */
+	void* hip_get_stream(mlContext_t context);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* MINML_HIP_BACKEND_H_ */

@@ -1,0 +1,407 @@
+"""Host-side mirror of the part of minml's core that drives the convolution / GEMM path on a device backend.
+
+`Context`, `Tensor` and the free functions below have the names, argument order and meaning of the reference's
+include/minml/core/{Context,Tensor,math}.hpp (dispatch: src/core/math.cpp, DeviceType::CUDA branch), so that tests written against
+them read like the reference's own tests (test/backend/test_winograd.cpp, test_conv2D.cpp, test_gemms.cpp, test_quantization.cpp).
+Every function converts its tensors to the by-value descriptors of the C-ABI and calls libminml_hip.so; nothing is computed here.
+
+Where the reference asserts (shape / dtype / device agreement) these functions raise ValueError *before* calling the library, because
+the library reports errors the reference's way, by C++ exceptions across the C boundary, which cannot be caught from Python.
+"""
+import ctypes
+
+import numpy as np
+
+from . import backend as B
+
+_NP_OF = {B.DTYPE_FLOAT16: np.uint16, B.DTYPE_FLOAT32: np.float32, B.DTYPE_INT8: np.int8, B.DTYPE_INT32: np.int32, B.DTYPE_UINT8: np.uint8}
+_NAME_OF = {"float16": B.DTYPE_FLOAT16, "float32": B.DTYPE_FLOAT32, "int8": B.DTYPE_INT8, "int32": B.DTYPE_INT32, "uint8": B.DTYPE_UINT8}
+ACTIVATIONS = {"linear": B.ACTIVATION_LINEAR, "sigmoid": B.ACTIVATION_SIGMOID, "tanh": B.ACTIVATION_TANH, "relu": B.ACTIVATION_RELU,
+               "leaky_relu": B.ACTIVATION_LEAKY_RELU, "exp": B.ACTIVATION_EXP, "gelu": B.ACTIVATION_EXP}
+
+
+def dtype_of(x):
+    if isinstance(x, str):
+        return _NAME_OF[x]
+    return int(x)
+
+
+def act_of(a):
+    if isinstance(a, str):
+        return ACTIVATIONS[a]
+    return int(a)
+
+
+def number_of_devices():
+    return B.fn("get_number_of_devices")()
+
+
+class Context:
+    """One stream on one device (reference: include/minml/core/Context.hpp; backend object src/backend/cuda/utils.hpp:28-66)."""
+
+    def __init__(self, device_index=0):
+        n = number_of_devices()
+        if not (0 <= device_index < n):
+            raise RuntimeError("no HIP device %d (devices found: %d)" % (device_index, n))
+        self.device_index = device_index
+        self.handle = B.fn("create_context")(device_index)
+
+    def synchronize(self):
+        B.fn("synchronize_with_context")(self.handle)
+
+    def isReady(self):
+        return bool(B.fn("is_context_ready")(self.handle))
+
+    def stream(self):
+        return B.fn("get_stream")(self.handle)
+
+    def destroy(self):
+        if self.handle:
+            B.fn("destroy_context")(self.handle)
+            self.handle = None
+
+
+class Event:
+    """Recorded on creation (reference: include/minml/core/Event.hpp, src/backend/cuda/cuda_event.cpp)."""
+
+    def __init__(self, context):
+        self.handle = B.fn("create_event")(context.handle)
+
+    def synchronize(self):
+        B.fn("wait_for_event")(self.handle)
+
+    def isReady(self):
+        return bool(B.fn("is_event_ready")(self.handle))
+
+    @staticmethod
+    def getElapsedTime(start, end):
+        return B.fn("get_time_between_events")(start.handle, end.handle)
+
+    def destroy(self):
+        if self.handle:
+            B.fn("destroy_event")(self.handle)
+            self.handle = None
+
+
+class Tensor:
+    """Dense row-major device tensor: pointer + shape + dtype + ownership flag (reference: src/core/Tensor.cpp, ml_memory.cpp:135-177).
+
+    fp16 data crosses the host boundary as numpy uint16 bit patterns.
+    """
+
+    def __init__(self, shape, dtype, device_index=0, _ptr=None, _owner=None):
+        self.shape = tuple(int(d) for d in shape)
+        self.dtype = dtype_of(dtype)
+        self.device_index = device_index
+        self._owner = _owner
+        if _ptr is None:
+            self.ptr = B.fn("malloc")(device_index, max(self.sizeInBytes(), 1))
+            self._owning = True
+        else:
+            self.ptr = _ptr
+            self._owning = False
+
+    # ---- shape helpers named as in the reference's Shape / Tensor
+    def rank(self):
+        return len(self.shape)
+
+    def dim(self, i):
+        return self.shape[i]
+
+    def volume(self):
+        v = 1
+        for d in self.shape:
+            v *= d
+        return v if self.shape else 0
+
+    def firstDim(self):
+        return self.shape[0]
+
+    def lastDim(self):
+        return self.shape[-1]
+
+    def sizeInBytes(self):
+        return self.volume() * B.DTYPE_SIZE[self.dtype]
+
+    def isEmpty(self):
+        return self.volume() == 0
+
+    def view(self, shape, offset=0):
+        """Non-owning tensor over the same memory, `offset` in elements (reference: Tensor::view)."""
+        shape = tuple(int(d) for d in shape)
+        vol = int(np.prod(shape)) if shape else 0
+        if offset + vol > self.volume():
+            raise ValueError("view exceeds the tensor")
+        p = B.fn("create_view")(self.ptr, offset * B.DTYPE_SIZE[self.dtype], vol * B.DTYPE_SIZE[self.dtype])
+        return Tensor(shape, self.dtype, self.device_index, _ptr=p, _owner=self)
+
+    def reinterpretAs(self, dtype):
+        """Same bytes, other element type; the last dimension is rescaled (used for the int32 view of the workspace)."""
+        new = dtype_of(dtype)
+        nbytes = self.sizeInBytes()
+        if nbytes % B.DTYPE_SIZE[new] != 0:
+            raise ValueError("size is not a multiple of the new element size")
+        return Tensor((nbytes // B.DTYPE_SIZE[new],), new, self.device_index, _ptr=self.ptr, _owner=self)
+
+    # ---- host <-> device
+    def copyFromHost(self, context, array):
+        arr = np.ascontiguousarray(array)
+        if arr.dtype != _NP_OF[self.dtype] or arr.size != self.volume():
+            raise ValueError("host array does not match tensor (dtype %s size %d vs %s %d)" % (arr.dtype, arr.size, _NP_OF[self.dtype], self.volume()))
+        if arr.size:
+            B.fn("memcpy_from_host")(context.handle if context else None, self.ptr, 0, arr.ctypes.data_as(ctypes.c_void_p), arr.nbytes)
+            if context is not None:
+                context.synchronize()  # the host array may go away
+        return self
+
+    def copyToHost(self, context=None):
+        out = np.empty(self.shape, _NP_OF[self.dtype])
+        if out.size:
+            if context is not None:
+                context.synchronize()
+            B.fn("memcpy_to_host")(None, out.ctypes.data_as(ctypes.c_void_p), self.ptr, 0, out.nbytes)
+        return out
+
+    def zeroall(self, context=None):
+        if self.sizeInBytes():
+            B.fn("memset")(context.handle if context else None, self.ptr, 0, self.sizeInBytes(), None, 0)
+
+    def setall(self, context, value):
+        pattern = np.array([value], _NP_OF[self.dtype]) if self.dtype != B.DTYPE_FLOAT16 else np.array([value], np.float16).view(np.uint16)
+        if self.sizeInBytes():
+            B.fn("memset")(context.handle if context else None, self.ptr, 0, self.sizeInBytes(), pattern.ctypes.data_as(ctypes.c_void_p),
+                           pattern.nbytes)
+
+    def free(self):
+        if self._owning and self.ptr:
+            B.fn("free")(self.ptr)
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+    # ---- descriptors
+    def desc(self):
+        return B.make_tensor(self.ptr, self.dtype, self.shape)
+
+    def shape_desc(self):
+        return B.make_shape(self.shape)
+
+
+def toDevice(context, array, dtype=None):
+    """numpy array -> new device tensor (uint16 arrays are fp16 bit patterns)."""
+    arr = np.ascontiguousarray(array)
+    if dtype is None:
+        dtype = {np.dtype(np.uint16): B.DTYPE_FLOAT16, np.dtype(np.float32): B.DTYPE_FLOAT32, np.dtype(np.int8): B.DTYPE_INT8,
+                 np.dtype(np.int32): B.DTYPE_INT32, np.dtype(np.uint8): B.DTYPE_UINT8}[arr.dtype]
+    t = Tensor(arr.shape, dtype, context.device_index)
+    t.copyFromHost(context, arr)
+    return t
+
+
+_EMPTY = B.make_tensor(None, B.DTYPE_UNKNOWN, ())
+
+
+def _desc(t):
+    return _EMPTY if (t is None or t.isEmpty()) else t.desc()
+
+
+def _ptr(t):
+    return None if (t is None or t.isEmpty()) else t.ptr
+
+
+def _require(cond, msg):
+    if not cond:
+        raise ValueError(msg)
+
+
+def _same_dtype(*tensors):
+    ts = [t for t in tensors if t is not None and not t.isEmpty()]
+    return all(t.dtype == ts[0].dtype for t in ts)
+
+
+def get_winograd_tile(weight_shape, matrices_shape):
+    """reference: src/core/math.cpp:107-118 — the tile size is derived from the number of matrices."""
+    _require(weight_shape[1] == weight_shape[2], "only square filters")
+    root = int(round(matrices_shape[0] ** 0.5))
+    _require(root * root == matrices_shape[0], "number of Winograd matrices is not a square")
+    return root - (weight_shape[1] - 1)
+
+
+def _require_winograd_supported(tile, kernel, dtype):
+    if not (tile == 4 and kernel == 3 and dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32)):
+        raise RuntimeError("No suitable Winograd transform runtime")  # reference: src/backend/cpu/winograd/winograd_runtime.cpp:516
+
+
+def winogradWeightTransform(context, weights, matrices, invert=False):
+    tile = get_winograd_tile(weights.shape, matrices.shape)
+    _require_winograd_supported(tile, weights.shape[1], weights.dtype)
+    _require(_same_dtype(weights, matrices), "dtype mismatch")
+    _require(matrices.shape == (36, weights.shape[0], weights.shape[3]), "matrices must be [36, Cout, Cin]")
+    B.fn("winograd_weight_transform")(context.handle, tile, weights.desc(), matrices.desc(), bool(invert))
+
+
+def winogradInputTransform(context, weight_shape, input, matrices):
+    tile = get_winograd_tile(weight_shape, matrices.shape)
+    _require_winograd_supported(tile, weight_shape[1], input.dtype)
+    _require(_same_dtype(input, matrices), "dtype mismatch")
+    b, h, w, c = input.shape
+    _require(matrices.shape == (36, b * ((h + 3) // 4) * ((w + 3) // 4), c), "matrices must be [36, tiles, C]")
+    B.fn("winograd_input_transform")(context.handle, tile, input.desc(), matrices.desc())
+
+
+def winogradOutputTransform(context, weight_shape, matrices, output, bias, add, act):
+    tile = get_winograd_tile(weight_shape, matrices.shape)
+    _require_winograd_supported(tile, weight_shape[1], output.dtype)
+    _require(_same_dtype(matrices, output, bias, add), "dtype mismatch")
+    b, h, w, c = output.shape
+    _require(matrices.shape == (36, b * ((h + 3) // 4) * ((w + 3) // 4), c), "matrices must be [36, tiles, C]")
+    _require(bias is None or bias.isEmpty() or bias.volume() == c, "bias must be [C]")
+    _require(add is None or add.isEmpty() or add.shape == output.shape, "add must have the output's shape")
+    B.fn("winograd_output_transform")(context.handle, tile, matrices.desc(), _desc(bias), _desc(add), output.desc(), act_of(act))
+
+
+def _gemm_dims(opA, A, opB, Bm):
+    ta, tb = opA in "tT", opB in "tT"
+    _require(opA in "ntNT" and opB in "ntNT", "op must be n or t")
+    M = A.shape[-1] if ta else A.shape[-2]
+    K = A.shape[-2] if ta else A.shape[-1]
+    N = Bm.shape[-2] if tb else Bm.shape[-1]
+    Kb = Bm.shape[-1] if tb else Bm.shape[-2]
+    _require(K == Kb, "inner dimensions differ")
+    return M, N, K
+
+
+def gemm(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
+    """C = alpha op(A) op(B) + beta C; an int32 C selects the int8 product (reference: src/core/math.cpp:643-660)."""
+    _require(A.rank() == 2 and Bm.rank() == 2 and C.rank() == 2, "gemm takes matrices")
+    M, N, K = _gemm_dims(opA, A, opB, Bm)
+    _require(C.shape == (M, N), "shape of C")
+    if C.dtype == B.DTYPE_INT32:
+        _require(A.dtype == B.DTYPE_INT8 and Bm.dtype == B.DTYPE_INT8 and alpha == 1.0 and beta == 0.0, "int8 product: int8 operands, alpha 1, beta 0")
+    else:
+        _require(_same_dtype(A, Bm, C) and C.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
+    B.fn("gemm_v2")(context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
+
+
+def gemmBatched(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
+    """reference: src/core/math.cpp:662-680; rank-2 operands are broadcast over the batch."""
+    _require(C.rank() == 3 and (A.rank() == 3 or Bm.rank() == 3), "gemmBatched takes rank-3 tensors")
+    M, N, K = _gemm_dims(opA, A, opB, Bm)
+    _require(C.shape[1:] == (M, N), "shape of C")
+    _require(A.rank() == 2 or A.shape[0] == C.shape[0], "batch of A")
+    _require(Bm.rank() == 2 or Bm.shape[0] == C.shape[0], "batch of B")
+    _require(_same_dtype(A, Bm, C) and C.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
+    B.fn("gemm_batched_v2")(context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
+
+
+def gemm_ex(context, D, alpha, opA, A, opB, Bm, beta, C, bias, act):
+    """D = act(alpha op(A) op(B) + beta C + bias) (reference: src/core/math.cpp:682-702)."""
+    M, N, K = _gemm_dims(opA, A, opB, Bm)
+    _require(D.shape == (M, N), "shape of D")
+    _require(beta == 0.0 or (C is not None and C.shape == (M, N)), "shape of C")
+    _require(_same_dtype(A, Bm, C, D, bias) and D.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
+    _require(bias is None or bias.isEmpty() or bias.volume() == N, "bias must be [N]")
+    c = C if (C is not None and not C.isEmpty()) else D
+    B.fn("gemm_ex")(context.handle, D.dtype, D.shape_desc(), D.ptr, alpha, opA.encode(), A.shape_desc(), A.ptr, opB.encode(), Bm.shape_desc(), Bm.ptr,
+                    beta, c.shape_desc(), c.ptr, _ptr(bias), act_of(act))
+
+
+def im2row(context, output, input, kernel_size, invert=False, padding=None):
+    """reference: src/core/math.cpp (im2row) -> cuda_im2row; `padding` is one host value or None for zeros."""
+    b, h, w, c = input.shape
+    _require(output.volume() == b * h * w * kernel_size * kernel_size * c, "im2row output size")
+    pad = None
+    if padding is not None:
+        pad = np.array([padding], _NP_OF[input.dtype])
+    B.fn("im2row")(context.handle, input.dtype, input.shape_desc(), output.ptr, input.ptr, kernel_size, bool(invert),
+                   None if pad is None else pad.ctypes.data_as(ctypes.c_void_p))
+
+
+def convolutionImplicitGemmForward(context, input, weights, output, bias, add, act):
+    """y = act(conv(x, w) + bias + add) (reference: src/core/math.cpp:399-416)."""
+    _require(input.rank() == 4 and weights.rank() == 4 and output.rank() == 4, "NHWC tensors")
+    _require(input.shape[3] == weights.shape[3] and output.shape[3] == weights.shape[0], "filters mismatch")
+    _require(output.shape[:3] == input.shape[:3], "stride 1, same padding")
+    _require(_same_dtype(input, weights, output, bias, add) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
+    _require(add is None or add.isEmpty() or add.shape == output.shape, "add must have the output's shape")
+    B.fn("convolution_implicit_gemm_forward")(context.handle, weights.dtype, input.shape_desc(), weights.shape_desc(), input.ptr, weights.ptr,
+                                              output.ptr, _ptr(bias), _ptr(add), act_of(act))
+
+
+def explicit_gemm_forward(context, input, output, weights, bias, workspace, activation, add=None):
+    """im2row + gemm_ex('n','t'), exactly the reference's sequence (src/core/math.cpp:1595-1626)."""
+    k = weights.shape[1]
+    _require(weights.shape[1] == weights.shape[2], "square kernel")
+    rows = input.volume() // input.lastDim()
+    cols = weights.volume() // weights.firstDim()
+    if k == 1:
+        input_matrix = input.view((rows, input.lastDim()))
+    else:
+        input_matrix = workspace.view((rows, cols))
+        im2row(context, input_matrix, input, k, False, None)
+    output_matrix = output.view((rows, output.lastDim()))
+    weight_matrix = weights.view((weights.firstDim(), cols))
+    if add is None or add.isEmpty():
+        gemm_ex(context, output_matrix, 1.0, "n", input_matrix, "t", weight_matrix, 0.0, output_matrix, bias, activation)
+    else:
+        gemm_ex(context, output_matrix, 1.0, "n", input_matrix, "t", weight_matrix, 1.0, add.view(output_matrix.shape), bias, activation)
+
+
+def quantized_scale_shift_act(context, output, output_transform, input, scales, bias, act, ext=None, ext_transform=(1.0, 0.0)):
+    """reference: src/core/math.cpp (quantized_scale_shift_act) -> cuda_quantized_scale_shift_act; transforms are (scale, shift)."""
+    _require(input.dtype == B.DTYPE_INT32 and scales.dtype == B.DTYPE_FLOAT32 and bias.dtype == B.DTYPE_FLOAT32, "int32 input, fp32 scales / bias")
+    _require(output.dtype in (B.DTYPE_INT8, B.DTYPE_FLOAT32, B.DTYPE_FLOAT16), "output must be int8, fp16 or fp32")
+    _require(input.volume() == output.volume() and scales.volume() == output.lastDim() and bias.volume() == output.lastDim(), "shape mismatch")
+    _require(ext is None or ext.isEmpty() or (ext.dtype == B.DTYPE_INT8 and ext.volume() == output.volume()), "ext must be int8 of the output's shape")
+    B.fn("quantized_scale_shift_act")(context.handle, output.dtype, output.shape_desc(), output.ptr, B.mlQuantizationData_t(*output_transform), input.ptr,
+                                      scales.ptr, bias.ptr, act_of(act), _ptr(ext), B.mlQuantizationData_t(*ext_transform))
+
+
+def quantizedConvForward(context, input, input_transform, weights, scales, bias, output, output_transform, ext=None, ext_transform=(1.0, 0.0),
+                         act="linear"):
+    """Whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 in one call (no counterpart in the reference's math.hpp)."""
+    _require(input.dtype == B.DTYPE_INT8 and weights.dtype == B.DTYPE_INT8, "int8 input and weights")
+    _require(input.shape[3] == weights.shape[3] and output.shape[3] == weights.shape[0] and output.shape[:3] == input.shape[:3], "shape mismatch")
+    _require(output.dtype in (B.DTYPE_INT8, B.DTYPE_FLOAT32), "output must be int8 or fp32")
+    _require(scales.volume() == weights.shape[0] and bias.volume() == weights.shape[0], "scales / bias must be [Cout]")
+    _require(ext is None or ext.isEmpty() or (ext.dtype == B.DTYPE_INT8 and ext.shape == output.shape), "ext must be int8 of the output's shape")
+    B.fn("quantized_conv_forward")(context.handle, input.shape_desc(), weights.shape_desc(), input.ptr, B.mlQuantizationData_t(*input_transform),
+                                   weights.ptr, scales.ptr, bias.ptr, output.dtype, output.ptr, B.mlQuantizationData_t(*output_transform), _ptr(ext),
+                                   B.mlQuantizationData_t(*ext_transform), act_of(act))
+
+
+def addBiasAct(context, alpha, input, bias, beta, output, act):
+    _require(_same_dtype(input, bias, output) and input.volume() == output.volume(), "shape / dtype mismatch")
+    _require(bias is None or bias.isEmpty() or bias.volume() == input.lastDim(), "bias must be [last dim]")
+    B.fn("add_bias_act")(context.handle, alpha, input.desc(), _desc(bias), beta, output.desc(), act_of(act))
+
+
+def activationForward(context, alpha, input, beta, output, act):
+    _require(_same_dtype(input, output) and input.volume() == output.volume(), "shape / dtype mismatch")
+    B.fn("activation_forward")(context.handle, alpha, input.desc(), beta, output.desc(), act_of(act))
+
+
+def addTensors(context, alpha1, x1, alpha2, x2, alpha3, x3, beta, y):
+    for x in (x1, x2, x3):
+        _require(x is None or x.isEmpty() or (x.volume() == y.volume() and x.dtype == y.dtype), "shape / dtype mismatch")
+    B.fn("add_tensors")(context.handle, alpha1, _desc(x1), alpha2, _desc(x2), alpha3, _desc(x3), beta, y.desc())
+
+
+def convertType(context, dst, src):
+    _require(dst.volume() == src.volume(), "size mismatch")
+    pair = (src.dtype, dst.dtype)
+    ok = src.dtype == dst.dtype or pair in ((B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), (B.DTYPE_FLOAT32, B.DTYPE_FLOAT16))
+    if not ok:
+        raise ValueError("unsupported conversion")  # reference: std::logic_error("unsupported conversion"), src/backend/cpu/dispatcher.cpp:61
+    B.fn("convert_type")(context.handle, dst.ptr, dst.dtype, src.ptr, src.dtype, src.volume())
+
+
+def unpackInput(context, dst, src):
+    """dst [..., C] <- bit planes packed 32 per uint32 word (reference: src/backend/cpu/dispatcher.cpp:112-123,143-174)."""
+    words = (dst.lastDim() + 31) // 32
+    _require(src.sizeInBytes() >= (dst.volume() // dst.lastDim()) * words * 4, "packed input too small")
+    B.fn("unpack_input")(context.handle, dst.shape_desc(), dst.dtype, dst.ptr, src.ptr)

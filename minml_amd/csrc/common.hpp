@@ -1,0 +1,157 @@
+/*
+ * common.hpp — shared host-side plumbing of the HIP backend: the context object behind mlContext_t, descriptor helpers
+ * and status checking. Counterpart of reference src/backend/cuda/utils.hpp:28-66 (Context{stream, workspace}) and
+ * include/minml/backend/backend_utils.hpp (size_of, volume, is_transpose).
+ */
+#ifndef MINML_AMD_COMMON_HPP_
+#define MINML_AMD_COMMON_HPP_
+
+#include "../../include/minml_hip_backend.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <cstddef>
+#include <stdexcept>
+#include <string>
+
+namespace mlhip
+{
+	struct Context
+	{
+			int device_index = 0;
+			hipStream_t stream = nullptr;
+			void *workspace = nullptr; /* lazily allocated device scratch owned by the context */
+			size_t workspace_size = 0;
+	};
+
+	struct Event
+	{
+			int device_index = 0;
+			hipEvent_t event = nullptr;
+	};
+
+	[[noreturn]] inline void fail_runtime(const std::string &msg)
+	{
+		throw std::runtime_error(msg);
+	}
+	[[noreturn]] inline void fail_logic(const std::string &msg)
+	{
+		throw std::logic_error(msg);
+	}
+
+	inline void check(hipError_t status, const char *what)
+	{
+		if (status != hipSuccess)
+			fail_runtime(std::string("HIP backend: ") + what + " failed: " + hipGetErrorString(status));
+	}
+#define MLHIP_CHECK(expr) ::mlhip::check((expr), #expr)
+#define MLHIP_REQUIRE(cond, msg) do { if (!(cond)) ::mlhip::fail_logic(std::string("HIP backend: ") + (msg)); } while (0)
+
+	inline Context* get(mlContext_t context)
+	{
+		if (context == nullptr)
+			fail_logic("HIP backend: null context");
+		return reinterpret_cast<Context*>(context);
+	}
+	inline hipStream_t stream_of(mlContext_t context)
+	{
+		return get(context)->stream;
+	}
+	/* returns device scratch of at least `bytes` bytes; grows by reallocating after the stream has drained */
+	void* get_workspace(mlContext_t context, size_t bytes);
+
+	inline int size_of(mlDataType_t dtype)
+	{
+		switch (dtype)
+		{
+			case DTYPE_FLOAT8:
+			case DTYPE_UINT8:
+			case DTYPE_INT8:
+				return 1;
+			case DTYPE_FLOAT16:
+			case DTYPE_INT16:
+				return 2;
+			case DTYPE_FLOAT32:
+			case DTYPE_INT32:
+				return 4;
+			case DTYPE_FLOAT64:
+				return 8;
+			default:
+				return 0;
+		}
+	}
+	inline size_t volume(const mlShape_t &s)
+	{
+		if (s.rank == 0)
+			return 0;
+		size_t result = 1;
+		for (int i = 0; i < s.rank; i++)
+			result *= static_cast<size_t>(s.dim[i]);
+		return result;
+	}
+	inline size_t volume(const mlTensor_t &t)
+	{
+		if (t.rank == 0)
+			return 0;
+		size_t result = 1;
+		for (int i = 0; i < t.rank; i++)
+			result *= static_cast<size_t>(t.dim[i]);
+		return result;
+	}
+	inline int last_dim(const mlTensor_t &t)
+	{
+		return (t.rank == 0) ? 0 : t.dim[t.rank - 1];
+	}
+	inline int last_dim(const mlShape_t &s)
+	{
+		return (s.rank == 0) ? 0 : s.dim[s.rank - 1];
+	}
+	inline mlShape_t shape_of(const mlTensor_t &t)
+	{
+		mlShape_t s;
+		s.rank = t.rank;
+		for (int i = 0; i < 6; i++)
+			s.dim[i] = t.dim[i];
+		return s;
+	}
+	inline mlTensor_t make_tensor(const void *data, mlDataType_t dtype, const mlShape_t &shape)
+	{
+		mlTensor_t t;
+		t.data = const_cast<void*>(data);
+		t.dtype = dtype;
+		t.rank = shape.rank;
+		for (int i = 0; i < 6; i++)
+			t.dim[i] = shape.dim[i];
+		return t;
+	}
+	inline bool is_transpose(char op)
+	{
+		if (op == 't' || op == 'T')
+			return true;
+		if (op == 'n' || op == 'N')
+			return false;
+		fail_logic("HIP backend: matrix op must be one of 'n', 'N', 't', 'T'");
+	}
+	template<typename T>
+	inline T* ptr(const mlTensor_t &t)
+	{
+		return reinterpret_cast<T*>(t.data);
+	}
+	inline int ceil_div(int a, int b)
+	{
+		return (a + b - 1) / b;
+	}
+} /* namespace mlhip */
+
+/*
+ * Exports hip_<name> a second time as cuda_<name>, the symbol minml's unmodified dispatcher calls for a device backend.
+ * An alias shares the definition, so both names have one address and one behaviour. Host pass only.
+ */
+#if defined(__HIP_DEVICE_COMPILE__)
+#define MLHIP_ALSO_AS_CUDA(name)
+#else
+#define MLHIP_ALSO_AS_CUDA(name) extern "C" __typeof__(hip_##name) cuda_##name __attribute__((alias("hip_" #name)));
+#endif
+
+#endif /* MINML_AMD_COMMON_HPP_ */

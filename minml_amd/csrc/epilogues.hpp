@@ -1,0 +1,233 @@
+/*
+ * epilogues.hpp — per-element tails applied to GEMM accumulators before they leave registers: the reference's fused
+ * "alpha, + bias, + beta*C, activation" (src/backend/cpu/gemm/def_kernels.cpp:237-275, avx512f_kernels.cpp:798-857) and the
+ * int8 requantisation of src/layers/Conv2D.cpp:284-306.
+ */
+#ifndef MINML_AMD_EPILOGUES_HPP_
+#define MINML_AMD_EPILOGUES_HPP_
+
+#include "device_utils.hpp"
+
+namespace mlhip
+{
+	/*
+	 * D[m][n] = act(alpha * acc + bias[n] + beta * C[m][n]); C is not read when beta == 0 (the Winograd workspace it may point to is
+	 * uninitialised). Activations other than LINEAR / RELU are applied to the value rounded to the storage type, because the reference
+	 * runs them as a second pass over the stored matrix (src/backend/cpu/gemm/gemm.cpp:81-82).
+	 */
+	template<typename T>
+	struct FloatEpilogue
+	{
+			T *D;
+			const T *C;
+			const T *bias;
+			int N; /* columns n >= N are not written */
+			int row_stride; /* elements between consecutive rows of C and D */
+			float alpha, beta;
+			int act;
+			bool vectorized; /* N % 4 == 0 and D, C, bias 4-element aligned */
+			static constexpr bool has_c = true;
+
+			__device__ __forceinline__ float finish(float x) const
+			{
+				if (act == ACTIVATION_RELU)
+					return fmaxf(x, 0.0f);
+				if (act != ACTIVATION_LINEAR)
+				{
+					if constexpr (sizeof(T) == 2)
+						x = half_bits_to_float(half_bits_rtz(x));
+					return activate(act, x);
+				}
+				return x;
+			}
+			__device__ __forceinline__ void operator()(int m, int n, const float (&acc)[4]) const
+			{
+				if (n >= N)
+					return;
+				const size_t offset = static_cast<size_t>(m) * row_stride + n;
+				if (vectorized)
+				{
+					Vec<T, 4> out;
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] = acc[e] * alpha;
+					if (bias != nullptr)
+					{
+						Vec<T, 4> b;
+						b.load(bias + n);
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							out.v[e] += b.v[e];
+					}
+					if (beta != 0.0f)
+					{
+						Vec<T, 4> c;
+						c.load(C + offset);
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							out.v[e] += beta * c.v[e];
+					}
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] = finish(out.v[e]);
+					out.store(D + offset);
+				}
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (n + e < N)
+						{
+							float x = acc[e] * alpha;
+							if (bias != nullptr)
+								x += Storage<T>::load(bias + n + e);
+							if (beta != 0.0f)
+								x += beta * Storage<T>::load(C + offset + e);
+							Storage<T>::store(D + offset + e, finish(x));
+						}
+				}
+			}
+	};
+
+	/* int8 x int8 -> int32 product stored as is (reference: src/backend/cuda/gemms.cpp:119-130, alpha = 1, beta = 0) */
+	struct Int32Epilogue
+	{
+			int32_t *D;
+			int N;
+			int row_stride;
+			bool vectorized;
+			static constexpr bool has_c = false;
+
+			__device__ __forceinline__ void operator()(int m, int n, const int (&acc)[4]) const
+			{
+				if (n >= N)
+					return;
+				const size_t offset = static_cast<size_t>(m) * row_stride + n;
+				if (vectorized)
+					*reinterpret_cast<int4_t*>(D + offset) = int4_t { acc[0], acc[1], acc[2], acc[3] };
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (n + e < N)
+							D[offset + e] = acc[e];
+				}
+			}
+	};
+
+	/*
+	 * The float tail of the reference's int8 convolution, evaluated in its order and without fused multiply-adds
+	 * (src/layers/Conv2D.cpp:284-306, include/minml/layers/quantization.hpp:39-47, src/layers/quantization.cpp:39-43):
+	 *   tmp = float(acc) * scale[n] + bias[n];  tmp += float(ext) * ext_scale + ext_shift;  tmp = act(tmp);
+	 *   q = clamp(round_half_away(tmp * inv_scale + inv_shift), -128, 127)      with inv_scale = 1 / out_scale, inv_shift = -out_shift / out_scale
+	 */
+	__device__ __forceinline__ float requant_value(int acc, float scale, float bias, bool has_ext, int ext, float ext_scale, float ext_shift, int act)
+	{
+#pragma clang fp contract(off)
+		float tmp = static_cast<float>(acc) * scale;
+		tmp = tmp + bias;
+		if (has_ext)
+		{
+			float e = static_cast<float>(ext) * ext_scale;
+			e = e + ext_shift;
+			tmp = tmp + e;
+		}
+		switch (act)
+		{
+			case ACTIVATION_SIGMOID:
+				tmp = 1.0f / (1.0f + expf(-tmp));
+				break;
+			case ACTIVATION_TANH:
+				tmp = tanhf(tmp);
+				break;
+			case ACTIVATION_RELU:
+				tmp = fmaxf(0.0f, tmp);
+				break;
+			case ACTIVATION_EXP:
+				tmp = expf(tmp);
+				break;
+			default:
+				break;
+		}
+		return tmp;
+	}
+	__device__ __forceinline__ int quantize_to_int8(float x, float inv_scale, float inv_shift)
+	{
+#pragma clang fp contract(off)
+		float q = x * inv_scale;
+		q = q + inv_shift;
+		q = roundf(q); /* half away from zero, as std::round */
+		q = fmaxf(-128.0f, fminf(127.0f, q));
+		return static_cast<int>(q);
+	}
+
+	template<typename OutT> /* int8_t (requantised), float or half_t (dequantised) */
+	struct RequantEpilogue
+	{
+			OutT *D;
+			const float *scales;
+			const float *bias;
+			const int8_t *ext;
+			int N;
+			int row_stride;
+			float ext_scale, ext_shift;
+			float inv_scale, inv_shift;
+			int act;
+			bool vectorized; /* N % 4 == 0 and all pointers 4-element aligned */
+			static constexpr bool has_c = false;
+
+			__device__ __forceinline__ void operator()(int m, int n, const int (&acc)[4]) const
+			{
+				if (n >= N)
+					return;
+				const size_t offset = static_cast<size_t>(m) * row_stride + n;
+				float vals[4];
+				if (vectorized)
+				{
+					const float4_t s = *reinterpret_cast<const float4_t*>(scales + n);
+					const float4_t b = *reinterpret_cast<const float4_t*>(bias + n);
+					uint32_t e_packed = 0;
+					if (ext != nullptr)
+						e_packed = *reinterpret_cast<const uint32_t*>(ext + offset);
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+					{
+						const int ext_val = static_cast<int>(static_cast<int8_t>((e_packed >> (8 * e)) & 0xffu));
+						vals[e] = requant_value(acc[e], s[e], b[e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+					}
+					if constexpr (sizeof(OutT) == 1)
+					{
+						uint32_t packed = 0;
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							packed |= (static_cast<uint32_t>(quantize_to_int8(vals[e], inv_scale, inv_shift)) & 0xffu) << (8 * e);
+						*reinterpret_cast<uint32_t*>(D + offset) = packed;
+					}
+					else
+					{
+						Vec<OutT, 4> out;
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							out.v[e] = vals[e];
+						out.store(D + offset);
+					}
+				}
+				else
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						if (n + e < N)
+						{
+							const int ext_val = (ext != nullptr) ? static_cast<int>(ext[offset + e]) : 0;
+							const float v = requant_value(acc[e], scales[n + e], bias[n + e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+							if constexpr (sizeof(OutT) == 1)
+								D[offset + e] = static_cast<OutT>(quantize_to_int8(v, inv_scale, inv_shift));
+							else
+								Storage<OutT>::store(D + offset + e, v);
+						}
+				}
+			}
+	};
+} /* namespace mlhip */
+
+#endif /* MINML_AMD_EPILOGUES_HPP_ */

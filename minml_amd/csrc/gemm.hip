@@ -1,0 +1,295 @@
+/*
+ * gemm.hip — GEMM entry points of the HIP backend: gemm / gemm_batched (both descriptor styles) and gemm_ex.
+ *
+ * Semantics follow the reference CPU backend (src/backend/cpu/gemm/gemm.cpp:34-83):
+ *   gemm:          C = alpha * op(A) * op(B) + beta * C
+ *   gemm_batched:  the same for every leading index; a rank-2 operand is broadcast (batch stride 0, gemm.cpp:18-29)
+ *   gemm_ex:       D = act(alpha * op(A) * op(B) + bias + beta * C), one dtype for A, B, C, D and bias, fp32 arithmetic
+ *   C.dtype INT32: int8 x int8 -> int32, alpha = 1, beta = 0 (src/backend/cuda/gemms.cpp:119-130)
+ * M, N, K are derived from the shapes as in src/backend/cpu/gemm/gemm_runtime.cpp:352-354.
+ *
+ * The inference path only ever asks for op(A) = 'n', op(B) = 't' (both operands K-contiguous): that case runs on the MFMA tile
+ * engine. Everything else (transposed forms used by training, K rows that are not 16-byte multiples, unaligned pointers) goes to
+ * a plain one-thread-per-output kernel that is correct for every case and makes no performance claim.
+ */
+#include "common.hpp"
+#include "gemm_core.hpp"
+#include "epilogues.hpp"
+#include "gemm_launch.hpp"
+
+namespace
+{
+	using namespace mlhip;
+
+	template<typename T, typename Cfg, typename Epilogue>
+	__global__ __launch_bounds__(Cfg::THREADS) void kernel_gemm_nt(const T *A, const T *B, int M, int N, int k_bytes, size_t stride_a,
+			size_t stride_b, size_t stride_c, Epilogue epilogue, int tiles_n)
+	{
+		__shared__ __attribute__((aligned(16))) uint8_t lds[Cfg::LDS_BYTES];
+
+		const unsigned int linear = xcd_contiguous_block_id(blockIdx.x, gridDim.x);
+		const int tile_m = linear / tiles_n;
+		const int tile_n = linear % tiles_n;
+		const size_t batch = blockIdx.y;
+
+		DenseRows<T> a_loader { A + batch * stride_a, M, k_bytes };
+		DenseRows<T> b_loader { B + batch * stride_b, N, k_bytes };
+		Epilogue local = epilogue;
+		local.D += batch * stride_c;
+		if constexpr (Epilogue::has_c)
+			local.C += batch * stride_c;
+		gemm_tile<T, Cfg>(a_loader, b_loader, M, k_bytes, tile_m * Cfg::BM, tile_n * Cfg::BN, lds, local);
+	}
+
+	/* Fallback: one thread per output element, any op combination, any alignment. */
+	template<typename T, typename AccT, typename Epilogue>
+	__global__ __launch_bounds__(256) void kernel_gemm_generic(const T *A, const T *B, int M, int N, int K, size_t a_row, size_t a_col, size_t b_row,
+			size_t b_col, size_t stride_a, size_t stride_b, size_t stride_c, Epilogue epilogue)
+	{
+		const size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+		if (gid >= static_cast<size_t>(M) * N)
+			return;
+		const int m = static_cast<int>(gid / N);
+		const int n = static_cast<int>(gid % N);
+		const size_t batch = blockIdx.y;
+		const T *a = A + batch * stride_a + m * a_row;
+		const T *b = B + batch * stride_b + n * b_row;
+		AccT acc = 0;
+		for (int k = 0; k < K; k++)
+		{
+			if constexpr (sizeof(T) == 1)
+				acc += static_cast<int>(a[k * a_col]) * static_cast<int>(b[k * b_col]);
+			else
+				acc += static_cast<float>(a[k * a_col]) * static_cast<float>(b[k * b_col]);
+		}
+		Epilogue local = epilogue;
+		local.D += batch * stride_c;
+		if constexpr (Epilogue::has_c)
+			local.C += batch * stride_c;
+		local.vectorized = false;
+		/* hand the single value over as the first of a group of 4 whose other members lie outside the matrix */
+		Epilogue single = local;
+		const AccT vals[4] = { acc, 0, 0, 0 };
+		single.N = n + 1;
+		single.row_stride = N;
+		single(m, n, vals);
+	}
+
+	bool aligned_to(const void *p, size_t bytes)
+	{
+		return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+	}
+}
+
+namespace mlhip
+{
+	void launch_gemm(hipStream_t stream, const GemmArgs &g)
+	{
+		if (g.M == 0 || g.N == 0 || g.batch == 0)
+			return;
+		MLHIP_REQUIRE(g.A != nullptr && g.B != nullptr && g.D != nullptr, "gemm: null matrix");
+		MLHIP_REQUIRE(g.beta == 0.0f || g.C != nullptr, "gemm: beta != 0 needs a C matrix");
+		MLHIP_REQUIRE(g.batch <= 65535, "gemm: at most 65535 matrices in a batch");
+
+		const int esize = size_of(g.dtype);
+		const bool nt = !g.transpose_a && g.transpose_b;
+		const size_t k_bytes = static_cast<size_t>(g.K) * esize;
+		const bool fast = nt && g.K > 0 && (k_bytes % 16 == 0) && aligned_to(g.A, 16) && aligned_to(g.B, 16)
+				&& ((g.stride_a * esize) % 16 == 0) && ((g.stride_b * esize) % 16 == 0);
+
+		const int out_size = (g.dtype == DTYPE_INT8) ? 4 : esize;
+		const bool vectorized = (g.N % 4 == 0) && aligned_to(g.D, 4 * out_size) && aligned_to(g.C, 4 * out_size) && aligned_to(g.bias, 4 * esize)
+				&& ((g.stride_c * out_size) % (4 * out_size) == 0);
+
+		/* strides of op(A)[m][k] and op(B)^T[n][k] in elements, for the generic kernel */
+		const size_t a_row = g.transpose_a ? 1 : g.K, a_col = g.transpose_a ? g.M : 1;
+		const size_t b_row = g.transpose_b ? g.K : 1, b_col = g.transpose_b ? 1 : g.N;
+
+		typedef TileConfig<128, 128, 64, 2, 2> Cfg;
+		const int tiles_m = ceil_div(g.M, Cfg::BM), tiles_n = ceil_div(g.N, Cfg::BN);
+		const dim3 fast_grid(static_cast<unsigned int>(tiles_m) * tiles_n, g.batch);
+		const size_t outputs = static_cast<size_t>(g.M) * g.N;
+		MLHIP_REQUIRE((outputs + 255) / 256 <= 0x7fffffffu, "gemm: matrix too large");
+		const dim3 slow_grid(static_cast<unsigned int>((outputs + 255) / 256), g.batch);
+
+		switch (g.dtype)
+		{
+			case DTYPE_FLOAT16:
+			{
+				FloatEpilogue<half_t> ep;
+				ep.D = reinterpret_cast<half_t*>(g.D);
+				ep.C = reinterpret_cast<const half_t*>(g.C);
+				ep.bias = reinterpret_cast<const half_t*>(g.bias);
+				ep.N = g.N;
+				ep.row_stride = g.N;
+				ep.alpha = g.alpha;
+				ep.beta = g.beta;
+				ep.act = g.act;
+				ep.vectorized = vectorized;
+				if (fast)
+					hipLaunchKernelGGL((kernel_gemm_nt<half_t, Cfg, FloatEpilogue<half_t>>), fast_grid, dim3(Cfg::THREADS), 0, stream,
+							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
+							g.stride_b, g.stride_c, ep, tiles_n);
+				else
+					hipLaunchKernelGGL((kernel_gemm_generic<half_t, float, FloatEpilogue<half_t>>), slow_grid, dim3(256), 0, stream,
+							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
+							g.stride_b, g.stride_c, ep);
+				break;
+			}
+			case DTYPE_FLOAT32:
+			{
+				FloatEpilogue<float> ep;
+				ep.D = reinterpret_cast<float*>(g.D);
+				ep.C = reinterpret_cast<const float*>(g.C);
+				ep.bias = reinterpret_cast<const float*>(g.bias);
+				ep.N = g.N;
+				ep.row_stride = g.N;
+				ep.alpha = g.alpha;
+				ep.beta = g.beta;
+				ep.act = g.act;
+				ep.vectorized = vectorized;
+				if (fast)
+					hipLaunchKernelGGL((kernel_gemm_nt<float, Cfg, FloatEpilogue<float>>), fast_grid, dim3(Cfg::THREADS), 0, stream,
+							reinterpret_cast<const float*>(g.A), reinterpret_cast<const float*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
+							g.stride_b, g.stride_c, ep, tiles_n);
+				else
+					hipLaunchKernelGGL((kernel_gemm_generic<float, float, FloatEpilogue<float>>), slow_grid, dim3(256), 0, stream,
+							reinterpret_cast<const float*>(g.A), reinterpret_cast<const float*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
+							g.stride_b, g.stride_c, ep);
+				break;
+			}
+			case DTYPE_INT8:
+			{
+				MLHIP_REQUIRE(g.bias == nullptr && g.act == ACTIVATION_LINEAR, "gemm: the int8 product has no fused epilogue");
+				Int32Epilogue ep;
+				ep.D = reinterpret_cast<int32_t*>(g.D);
+				ep.N = g.N;
+				ep.row_stride = g.N;
+				ep.vectorized = vectorized;
+				if (fast)
+					hipLaunchKernelGGL((kernel_gemm_nt<int8_t, Cfg, Int32Epilogue>), fast_grid, dim3(Cfg::THREADS), 0, stream,
+							reinterpret_cast<const int8_t*>(g.A), reinterpret_cast<const int8_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
+							g.stride_b, g.stride_c, ep, tiles_n);
+				else
+					hipLaunchKernelGGL((kernel_gemm_generic<int8_t, int, Int32Epilogue>), slow_grid, dim3(256), 0, stream,
+							reinterpret_cast<const int8_t*>(g.A), reinterpret_cast<const int8_t*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
+							g.stride_b, g.stride_c, ep);
+				break;
+			}
+			default:
+				fail_logic("HIP backend: gemm: unsupported data type");
+		}
+		MLHIP_CHECK(hipGetLastError());
+	}
+
+	GemmArgs make_gemm_args(mlDataType_t dtype, char opA, char opB, const mlShape_t &shape_A, const mlShape_t &shape_B, const mlShape_t &shape_D,
+			bool batched)
+	{
+		GemmArgs g;
+		g.dtype = dtype;
+		g.transpose_a = is_transpose(opA);
+		g.transpose_b = is_transpose(opB);
+		MLHIP_REQUIRE(shape_A.rank == 2 || shape_A.rank == 3, "gemm: A must have rank 2 or 3");
+		MLHIP_REQUIRE(shape_B.rank == 2 || shape_B.rank == 3, "gemm: B must have rank 2 or 3");
+		const int ar = shape_A.dim[shape_A.rank - 2], ac = shape_A.dim[shape_A.rank - 1];
+		const int br = shape_B.dim[shape_B.rank - 2], bc = shape_B.dim[shape_B.rank - 1];
+		g.M = g.transpose_a ? ac : ar;
+		g.K = g.transpose_a ? ar : ac;
+		g.N = g.transpose_b ? br : bc;
+		const int kb = g.transpose_b ? bc : br;
+		MLHIP_REQUIRE(kb == g.K, "gemm: inner dimensions of A and B differ");
+		if (batched)
+		{
+			MLHIP_REQUIRE(shape_D.rank == 3, "gemm_batched: C must have rank 3");
+			MLHIP_REQUIRE(shape_A.rank == 3 || shape_B.rank == 3, "gemm_batched: at least one of A, B must have rank 3");
+			g.batch = shape_D.dim[0];
+			if (shape_A.rank == 3)
+				MLHIP_REQUIRE(shape_A.dim[0] == g.batch, "gemm_batched: batch size of A differs from C");
+			if (shape_B.rank == 3)
+				MLHIP_REQUIRE(shape_B.dim[0] == g.batch, "gemm_batched: batch size of B differs from C");
+			g.stride_a = (shape_A.rank == 3) ? static_cast<size_t>(ar) * ac : 0;
+			g.stride_b = (shape_B.rank == 3) ? static_cast<size_t>(br) * bc : 0;
+			g.stride_c = static_cast<size_t>(shape_D.dim[1]) * shape_D.dim[2];
+			MLHIP_REQUIRE(shape_D.dim[1] == g.M && shape_D.dim[2] == g.N, "gemm_batched: shape of C does not match op(A) * op(B)");
+		}
+		else
+		{
+			MLHIP_REQUIRE(shape_A.rank == 2 && shape_B.rank == 2 && shape_D.rank == 2, "gemm: matrices must have rank 2");
+			g.batch = 1;
+			MLHIP_REQUIRE(shape_D.dim[0] == g.M && shape_D.dim[1] == g.N, "gemm: shape of the output does not match op(A) * op(B)");
+		}
+		return g;
+	}
+}
+
+extern "C"
+{
+	using namespace mlhip;
+
+	void hip_gemm(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
+			const void *B, char opA, char opB, float alpha, float beta)
+	{
+		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_C, false);
+		g.A = A;
+		g.B = B;
+		g.C = C;
+		g.D = C;
+		g.alpha = alpha;
+		g.beta = beta;
+		launch_gemm(stream_of(context), g);
+	}
+	void hip_gemm_batched(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
+			const void *B, char opA, char opB, float alpha, float beta)
+	{
+		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_C, true);
+		g.A = A;
+		g.B = B;
+		g.C = C;
+		g.D = C;
+		g.alpha = alpha;
+		g.beta = beta;
+		launch_gemm(stream_of(context), g);
+	}
+	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
+	{
+		mlDataType_t dtype = C.dtype;
+		if (C.dtype == DTYPE_INT32)
+		{
+			MLHIP_REQUIRE(A.dtype == DTYPE_INT8 && B.dtype == DTYPE_INT8, "gemm: an INT32 result needs INT8 operands");
+			MLHIP_REQUIRE(alpha == 1.0f && beta == 0.0f, "gemm: the int8 product supports alpha = 1, beta = 0 only");
+			dtype = DTYPE_INT8;
+		}
+		else
+			MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm: A, B and C must have one data type");
+		hip_gemm(context, dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
+	}
+	void hip_gemm_batched_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
+	{
+		MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm_batched: A, B and C must have one data type");
+		MLHIP_REQUIRE(C.dtype == DTYPE_FLOAT16 || C.dtype == DTYPE_FLOAT32, "gemm_batched: unsupported data type");
+		hip_gemm_batched(context, C.dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
+	}
+	void hip_gemm_ex(mlContext_t context, mlDataType_t dtype, mlShape_t shape_D, void *D, float alpha, char opA, mlShape_t shape_A, const void *A,
+			char opB, mlShape_t shape_B, const void *B, float beta, mlShape_t shape_C, const void *C, const void *bias, mlActivationType_t act)
+	{
+		MLHIP_REQUIRE(dtype == DTYPE_FLOAT16 || dtype == DTYPE_FLOAT32, "gemm_ex: unsupported data type");
+		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_D, false);
+		if (beta != 0.0f)
+			MLHIP_REQUIRE(shape_C.rank == 2 && shape_C.dim[0] == g.M && shape_C.dim[1] == g.N, "gemm_ex: C must have the shape of D");
+		g.A = A;
+		g.B = B;
+		g.C = C;
+		g.D = D;
+		g.alpha = alpha;
+		g.beta = beta;
+		g.bias = bias;
+		g.act = act;
+		launch_gemm(stream_of(context), g);
+	}
+} /* extern "C" */
+
+MLHIP_ALSO_AS_CUDA(gemm)
+MLHIP_ALSO_AS_CUDA(gemm_batched)
+MLHIP_ALSO_AS_CUDA(gemm_v2)
+MLHIP_ALSO_AS_CUDA(gemm_batched_v2)
+MLHIP_ALSO_AS_CUDA(gemm_ex)

@@ -1,0 +1,483 @@
+/*
+ * winograd.hip — Winograd F(4x4, 3x3) weight / input / output transforms for gfx950, NHWC, fp16 and fp32 storage, fp32 arithmetic.
+ *
+ * What they compute follows the reference CPU backend:
+ *   tile geometry, zero padding, matrix index order      src/backend/cpu/winograd/winograd_runtime.cpp:47-232
+ *   weight transform (columns first, then rows)          src/backend/cpu/winograd/def_winograd_kernels.cpp:165-184,380-424
+ *   input / output 1-D transforms incl. FMA placement    src/backend/cpu/winograd/avx2_winograd_kernels.cpp:241-279 (same in avx512f_*:241-279)
+ *   output epilogue order: + bias, + ext, ReLU           src/backend/cpu/winograd/avx2_winograd_kernels.cpp:611-622
+ *   other activations = separate pass over the stored y  src/backend/cpu/winograd/winograd_runtime.cpp:529-536
+ * The floating-point expression trees below are written to be evaluated exactly as the reference evaluates them (explicit fma
+ * where it uses one, no contraction elsewhere), so fp32 results and truncated fp16 results agree bit for bit.
+ *
+ * How they run: the transforms are pure streaming kernels (bound by HBM bandwidth). One thread owns VEC consecutive channels of one
+ * tile, so that a wavefront touches 64*VEC consecutive channels with one 4/8/16-byte access per lane; a 6x6 tile of
+ * VEC channels lives in registers. Neighbouring tiles of one image are placed on the same XCD so that the two rows / columns of
+ * halo they share are served by that XCD's L2.
+ */
+#include "common.hpp"
+#include "device_utils.hpp"
+
+#pragma clang fp contract(off)
+
+namespace
+{
+	using namespace mlhip;
+
+	/* ---------------------------------------------------------------------------------------------------------------------
+	 * 1-D transforms on VEC channels at once
+	 * ------------------------------------------------------------------------------------------------------------------- */
+	template<int VEC>
+	struct Line6
+	{
+			float v[6][VEC];
+	};
+	template<int VEC>
+	struct Line4
+	{
+			float v[4][VEC];
+	};
+
+	/* Bt * d, rows evaluated as  r0=(l0-l2)+c14(l4-l2)  r1=(l1+l2)-c14(l3+l4)  r2=(l2-l1)+c14(l3-l4)
+	 *                            r3=(l3-l1)+c12(l4-l2)  r4=(l1-l3)+c12(l4-l2)  r5=(l1-l3)+c14(l5-l3), last step fused */
+	template<int VEC>
+	__device__ __forceinline__ void input_transform_1d(const float (&l)[6][VEC], float (&r)[6][VEC])
+	{
+#pragma unroll
+		for (int c = 0; c < VEC; c++)
+		{
+			const float l0 = l[0][c], l1 = l[1][c], l2 = l[2][c], l3 = l[3][c], l4 = l[4][c], l5 = l[5][c];
+			r[0][c] = __builtin_fmaf(0.25f, l4 - l2, l0 - l2);
+			r[1][c] = __builtin_fmaf(-0.25f, l3 + l4, l1 + l2);
+			r[2][c] = __builtin_fmaf(0.25f, l3 - l4, l2 - l1);
+			r[3][c] = __builtin_fmaf(0.5f, l4 - l2, l3 - l1);
+			r[4][c] = __builtin_fmaf(0.5f, l4 - l2, l1 - l3);
+			r[5][c] = __builtin_fmaf(0.25f, l5 - l3, l1 - l3);
+		}
+	}
+	/* At * m:  s=l1+l2 d=l1-l2 p=l3+l4 q=l3-l4;  o0=(l0+s)+c14*p  o1=d+c12*q  o2=s+p  o3=(d+2*l5)+2*q */
+	template<int VEC>
+	__device__ __forceinline__ void output_transform_1d(const float (&l)[6][VEC], float (&o)[4][VEC])
+	{
+#pragma unroll
+		for (int c = 0; c < VEC; c++)
+		{
+			const float l0 = l[0][c], l1 = l[1][c], l2 = l[2][c], l3 = l[3][c], l4 = l[4][c], l5 = l[5][c];
+			const float s = l1 + l2;
+			const float d = l1 - l2;
+			const float p = l3 + l4;
+			const float q = l3 - l4;
+			o[0][c] = __builtin_fmaf(0.25f, p, l0 + s);
+			o[1][c] = __builtin_fmaf(0.5f, q, d);
+			o[2][c] = s + p;
+			o[3][c] = __builtin_fmaf(2.0f, q, __builtin_fmaf(2.0f, l5, d));
+		}
+	}
+	/* G * g with the constants rounded to fp32 and no fused operations */
+	__device__ __forceinline__ void weight_transform_1d(const float (&g)[3], float (&w)[6])
+	{
+		const float c13 = 1.0 / 3.0;
+		const float c23 = 2.0 / 3.0;
+		const float c43 = 4.0 / 3.0;
+		const float c2 = 2.0;
+		w[0] = g[0];
+		w[1] = c23 * ((g[0] + g[1]) + g[2]);
+		w[2] = c23 * ((g[0] - g[1]) + g[2]);
+		w[3] = (c13 * g[0] + c23 * g[1]) + c43 * g[2];
+		w[4] = (c13 * g[0] - c23 * g[1]) + c43 * g[2];
+		w[5] = c2 * g[2];
+	}
+
+	/* ---------------------------------------------------------------------------------------------------------------------
+	 * kernels
+	 * ------------------------------------------------------------------------------------------------------------------- */
+	/* weights [Cout][3][3][Cin] -> matrices [36][Cout][Cin]; one thread per (cout, cin) */
+	template<typename T>
+	__global__ __launch_bounds__(256) void kernel_weight_transform_4x4_3x3(const T *__restrict__ weights, T *__restrict__ matrices,
+			int filters_out, int filters_in, bool invert)
+	{
+		const size_t total = static_cast<size_t>(filters_out) * filters_in;
+		const size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+		if (gid >= total)
+			return;
+		const int out = static_cast<int>(gid / filters_in);
+		const int in = static_cast<int>(gid % filters_in);
+
+		float tile[3][3];
+#pragma unroll
+		for (int i = 0; i < 3; i++)
+#pragma unroll
+			for (int j = 0; j < 3; j++)
+			{
+				const int x = invert ? (2 - i) : i;
+				const int y = invert ? (2 - j) : j;
+				tile[i][j] = Storage<T>::load(weights + ((static_cast<size_t>(out) * 3 + x) * 3 + y) * filters_in + in);
+			}
+
+		float tmp[6][3]; /* columns first */
+#pragma unroll
+		for (int col = 0; col < 3; col++)
+		{
+			const float g[3] = { tile[0][col], tile[1][col], tile[2][col] };
+			float w[6];
+			weight_transform_1d(g, w);
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+				tmp[row][col] = w[row];
+		}
+#pragma unroll
+		for (int row = 0; row < 6; row++)
+		{
+			float w[6];
+			weight_transform_1d(tmp[row], w);
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+				Storage<T>::store(matrices + (static_cast<size_t>(row * 6 + col) * filters_out + out) * filters_in + in, w[col]);
+		}
+	}
+
+	/* input [B][H][W][C] -> matrices [36][B*tiles_h*tiles_w][C] */
+	template<typename T, int VEC>
+	__global__ __launch_bounds__(256) void kernel_input_transform_4x4_3x3(const T *__restrict__ input, T *__restrict__ matrices, int batch_size,
+			int height, int width, int channels, int tiles_h, int tiles_w)
+	{
+		const int groups = channels / VEC;
+		const int tiles_per_image = tiles_h * tiles_w;
+		const size_t nb_of_tiles = static_cast<size_t>(batch_size) * tiles_per_image;
+		const size_t total = nb_of_tiles * groups;
+
+		const unsigned int block = xcd_contiguous_block_id(blockIdx.x, gridDim.x);
+		const size_t gid = static_cast<size_t>(block) * blockDim.x + threadIdx.x;
+		if (gid >= total)
+			return;
+		const size_t tile_idx = gid / groups;
+		const int channel = static_cast<int>(gid % groups) * VEC;
+
+		const int batch = static_cast<int>(tile_idx / tiles_per_image);
+		const int in_image = static_cast<int>(tile_idx % tiles_per_image);
+		const int x0 = 4 * (in_image / tiles_w) - 1;
+		const int y0 = 4 * (in_image % tiles_w) - 1;
+
+		const T *src = input + static_cast<size_t>(batch) * height * width * channels + channel;
+
+		float tmp[6][6][VEC]; /* [row after the column pass][col] */
+#pragma unroll
+		for (int col = 0; col < 6; col++)
+		{
+			const int y = y0 + col;
+			float line[6][VEC];
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+			{
+				const int x = x0 + row;
+				Vec<T, VEC> tmpv;
+				if (x >= 0 && x < height && y >= 0 && y < width)
+					tmpv.load(src + (static_cast<size_t>(x) * width + y) * channels);
+				else
+					tmpv.zero();
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
+					line[row][c] = tmpv.v[c];
+			}
+			float res[6][VEC];
+			input_transform_1d<VEC>(line, res);
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
+					tmp[row][col][c] = res[row][c];
+		}
+
+		T *dst = matrices + tile_idx * channels + channel;
+		const size_t matrix_stride = nb_of_tiles * channels;
+#pragma unroll
+		for (int row = 0; row < 6; row++)
+		{
+			float res[6][VEC];
+			input_transform_1d<VEC>(tmp[row], res);
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+			{
+				Vec<T, VEC> out;
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
+					out.v[c] = res[col][c];
+				out.store(dst + static_cast<size_t>(row * 6 + col) * matrix_stride);
+			}
+		}
+	}
+
+	/* matrices [36][B*tiles_h*tiles_w][C] (+ bias [C], + ext [B][H][W][C]) -> output [B][H][W][C] */
+	template<typename T, int VEC>
+	__global__ __launch_bounds__(256) void kernel_output_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+			const T *ext, int act, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
+	{
+		const int groups = channels / VEC;
+		const int tiles_per_image = tiles_h * tiles_w;
+		const size_t nb_of_tiles = static_cast<size_t>(batch_size) * tiles_per_image;
+		const size_t total = nb_of_tiles * groups;
+
+		const unsigned int block = xcd_contiguous_block_id(blockIdx.x, gridDim.x);
+		const size_t gid = static_cast<size_t>(block) * blockDim.x + threadIdx.x;
+		if (gid >= total)
+			return;
+		const size_t tile_idx = gid / groups;
+		const int channel = static_cast<int>(gid % groups) * VEC;
+
+		const int batch = static_cast<int>(tile_idx / tiles_per_image);
+		const int in_image = static_cast<int>(tile_idx % tiles_per_image);
+		const int x0 = 4 * (in_image / tiles_w);
+		const int y0 = 4 * (in_image % tiles_w);
+
+		const T *src = matrices + tile_idx * channels + channel;
+		const size_t matrix_stride = nb_of_tiles * channels;
+
+		float tmp[4][6][VEC];
+#pragma unroll
+		for (int col = 0; col < 6; col++)
+		{
+			float line[6][VEC];
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+			{
+				Vec<T, VEC> tmpv;
+				tmpv.load(src + static_cast<size_t>(row * 6 + col) * matrix_stride);
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
+					line[row][c] = tmpv.v[c];
+			}
+			float res[4][VEC];
+			output_transform_1d<VEC>(line, res);
+#pragma unroll
+			for (int row = 0; row < 4; row++)
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
+					tmp[row][col][c] = res[row][c];
+		}
+
+		Vec<T, VEC> b;
+		if (bias != nullptr)
+			b.load(bias + channel);
+		else
+			b.zero();
+
+		const size_t image_offset = static_cast<size_t>(batch) * height * width * channels + channel;
+#pragma unroll
+		for (int row = 0; row < 4; row++)
+		{
+			float res[4][VEC];
+			output_transform_1d<VEC>(tmp[row], res);
+			const int x = x0 + row;
+#pragma unroll
+			for (int col = 0; col < 4; col++)
+			{
+				const int y = y0 + col;
+				if (x < height && y < width)
+				{
+					const size_t offset = image_offset + (static_cast<size_t>(x) * width + y) * channels;
+					Vec<T, VEC> out;
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						out.v[c] = res[col][c] + b.v[c];
+					if (ext != nullptr)
+					{
+						Vec<T, VEC> e;
+						e.load(ext + offset);
+#pragma unroll
+						for (int c = 0; c < VEC; c++)
+							out.v[c] = out.v[c] + e.v[c];
+					}
+					if (act == ACTIVATION_RELU)
+					{
+#pragma unroll
+						for (int c = 0; c < VEC; c++)
+							out.v[c] = fmaxf(out.v[c], 0.0f);
+					}
+					else if (act != ACTIVATION_LINEAR)
+					{ /* the reference stores y and then runs the activation over it: round through the storage type in between */
+#pragma unroll
+						for (int c = 0; c < VEC; c++)
+						{
+							float t = out.v[c];
+							if constexpr (sizeof(T) == 2)
+								t = half_bits_to_float(half_bits_rtz(t));
+							out.v[c] = activate(act, t);
+						}
+					}
+					out.store(output + offset);
+				}
+			}
+		}
+	}
+
+	/* ---------------------------------------------------------------------------------------------------------------------
+	 * host side
+	 * ------------------------------------------------------------------------------------------------------------------- */
+	int integer_sqrt(int x)
+	{
+		int r = 0;
+		while ((r + 1) * (r + 1) <= x)
+			r++;
+		return r;
+	}
+	/* the kernel size is not an argument: matrices.dim[0] = (tile + kernel - 1)^2 (reference: src/core/math.cpp:107-118) */
+	void require_supported(int tile_size, const mlTensor_t &matrices, mlDataType_t dtype)
+	{
+		MLHIP_REQUIRE(matrices.rank == 3, "Winograd matrices must have rank 3");
+		const int transform = integer_sqrt(matrices.dim[0]);
+		const int kernel_size = transform + 1 - tile_size;
+		const bool ok = (transform * transform == matrices.dim[0]) && tile_size == 4 && kernel_size == 3
+				&& (dtype == DTYPE_FLOAT16 || dtype == DTYPE_FLOAT32);
+		if (!ok)
+			fail_runtime("No suitable Winograd transform runtime");
+	}
+	int pick_vec(int channels, const void *p0, const void *p1, const void *p2, const void *p3, int elem_size)
+	{
+		/* widest access is 16 bytes for fp32 (4 channels) and 8 bytes for fp16 (4 channels): 144 live fp32 values per thread */
+		int vec = 4;
+		while (vec > 1)
+		{
+			const uintptr_t bytes = static_cast<uintptr_t>(vec) * elem_size;
+			const bool aligned = (reinterpret_cast<uintptr_t>(p0) % bytes == 0) && (reinterpret_cast<uintptr_t>(p1) % bytes == 0)
+					&& (reinterpret_cast<uintptr_t>(p2) % bytes == 0) && (reinterpret_cast<uintptr_t>(p3) % bytes == 0);
+			if (channels % vec == 0 && aligned)
+				break;
+			vec /= 2;
+		}
+		return vec;
+	}
+	unsigned int grid_for(size_t threads)
+	{
+		const size_t blocks = (threads + 255) / 256;
+		MLHIP_REQUIRE(blocks <= 0x7fffffffu, "tensor too large for one launch");
+		return static_cast<unsigned int>(blocks);
+	}
+
+	template<typename T>
+	void launch_input(hipStream_t stream, const mlTensor_t &x, mlTensor_t &matrices)
+	{
+		const int batch = x.dim[0], height = x.dim[1], width = x.dim[2], channels = x.dim[3];
+		const int tiles_h = ceil_div(height, 4), tiles_w = ceil_div(width, 4);
+		const size_t tiles = static_cast<size_t>(batch) * tiles_h * tiles_w;
+		const int vec = pick_vec(channels, x.data, matrices.data, nullptr, nullptr, sizeof(T));
+		const dim3 block(256);
+		const dim3 grid(grid_for(tiles * (channels / vec)));
+		const T *in = ptr<const T>(x);
+		T *out = ptr<T>(matrices);
+		switch (vec)
+		{
+			case 4:
+				hipLaunchKernelGGL((kernel_input_transform_4x4_3x3<T, 4>), grid, block, 0, stream, in, out, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+			case 2:
+				hipLaunchKernelGGL((kernel_input_transform_4x4_3x3<T, 2>), grid, block, 0, stream, in, out, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+			default:
+				hipLaunchKernelGGL((kernel_input_transform_4x4_3x3<T, 1>), grid, block, 0, stream, in, out, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+		}
+		MLHIP_CHECK(hipGetLastError());
+	}
+	template<typename T>
+	void launch_output(hipStream_t stream, const mlTensor_t &matrices, const mlTensor_t &bias, const mlTensor_t &ext, mlTensor_t &y, mlActivationType_t act)
+	{
+		const int batch = y.dim[0], height = y.dim[1], width = y.dim[2], channels = y.dim[3];
+		const int tiles_h = ceil_div(height, 4), tiles_w = ceil_div(width, 4);
+		const size_t tiles = static_cast<size_t>(batch) * tiles_h * tiles_w;
+		const int vec = pick_vec(channels, matrices.data, y.data, bias.data, ext.data, sizeof(T));
+		const dim3 block(256);
+		const dim3 grid(grid_for(tiles * (channels / vec)));
+		const T *in = ptr<const T>(matrices);
+		T *out = ptr<T>(y);
+		const T *b = ptr<const T>(bias);
+		const T *e = ptr<const T>(ext);
+		const int a = static_cast<int>(act);
+		switch (vec)
+		{
+			case 4:
+				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 4>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+			case 2:
+				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 2>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+			default:
+				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 1>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				break;
+		}
+		MLHIP_CHECK(hipGetLastError());
+	}
+}
+
+extern "C"
+{
+	using namespace mlhip;
+
+	void hip_winograd_weight_transform(mlContext_t context, int tile_size, const mlTensor_t w, mlTensor_t matrices, bool invert)
+	{
+		hipStream_t stream = stream_of(context);
+		MLHIP_REQUIRE(w.rank == 4 && w.dim[1] == w.dim[2], "Winograd weights must be [Cout, k, k, Cin] with a square kernel");
+		require_supported(tile_size, matrices, w.dtype);
+		MLHIP_REQUIRE(w.dim[1] == 3, "Winograd weight transform: weight kernel size does not match the matrices");
+		MLHIP_REQUIRE(matrices.dtype == w.dtype, "Winograd weight transform: dtype mismatch");
+		MLHIP_REQUIRE(matrices.dim[1] == w.dim[0] && matrices.dim[2] == w.dim[3], "Winograd weight transform: matrices must be [36, Cout, Cin]");
+		MLHIP_REQUIRE(w.data != nullptr && matrices.data != nullptr, "Winograd weight transform: null tensor");
+
+		const size_t threads = static_cast<size_t>(w.dim[0]) * w.dim[3];
+		if (threads == 0)
+			return;
+		const dim3 block(256);
+		const dim3 grid(grid_for(threads));
+		if (w.dtype == DTYPE_FLOAT16)
+			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<half_t>, grid, block, 0, stream, ptr<const half_t>(w), ptr<half_t>(matrices), w.dim[0],
+					w.dim[3], invert);
+		else
+			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<float>, grid, block, 0, stream, ptr<const float>(w), ptr<float>(matrices), w.dim[0],
+					w.dim[3], invert);
+		MLHIP_CHECK(hipGetLastError());
+	}
+	void hip_winograd_input_transform(mlContext_t context, int tile_size, const mlTensor_t x, mlTensor_t matrices)
+	{
+		hipStream_t stream = stream_of(context);
+		MLHIP_REQUIRE(x.rank == 4, "Winograd input transform: input must be [B, H, W, C]");
+		require_supported(tile_size, matrices, x.dtype);
+		MLHIP_REQUIRE(matrices.dtype == x.dtype, "Winograd input transform: dtype mismatch");
+		const size_t tiles = static_cast<size_t>(x.dim[0]) * ceil_div(x.dim[1], 4) * ceil_div(x.dim[2], 4);
+		MLHIP_REQUIRE(static_cast<size_t>(matrices.dim[1]) == tiles && matrices.dim[2] == x.dim[3],
+				"Winograd input transform: matrices must be [36, B*ceil(H/4)*ceil(W/4), C]");
+		if (tiles == 0 || x.dim[3] == 0)
+			return;
+		MLHIP_REQUIRE(x.data != nullptr && matrices.data != nullptr, "Winograd input transform: null tensor");
+		mlTensor_t m = matrices;
+		if (x.dtype == DTYPE_FLOAT16)
+			launch_input<half_t>(stream, x, m);
+		else
+			launch_input<float>(stream, x, m);
+	}
+	void hip_winograd_output_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
+			mlTensor_t y, mlActivationType_t act)
+	{
+		hipStream_t stream = stream_of(context);
+		MLHIP_REQUIRE(y.rank == 4, "Winograd output transform: output must be [B, H, W, C]");
+		require_supported(tile_size, matrices, y.dtype);
+		MLHIP_REQUIRE(matrices.dtype == y.dtype, "Winograd output transform: dtype mismatch");
+		const size_t tiles = static_cast<size_t>(y.dim[0]) * ceil_div(y.dim[1], 4) * ceil_div(y.dim[2], 4);
+		MLHIP_REQUIRE(static_cast<size_t>(matrices.dim[1]) == tiles && matrices.dim[2] == y.dim[3],
+				"Winograd output transform: matrices must be [36, B*ceil(H/4)*ceil(W/4), C]");
+		if (bias.data != nullptr)
+			MLHIP_REQUIRE(bias.dtype == y.dtype && volume(bias) == static_cast<size_t>(y.dim[3]), "Winograd output transform: bias must be [C] of the output dtype");
+		if (ext.data != nullptr)
+			MLHIP_REQUIRE(ext.dtype == y.dtype && volume(ext) == volume(y), "Winograd output transform: ext must have the output's shape and dtype");
+		if (tiles == 0 || y.dim[3] == 0)
+			return;
+		MLHIP_REQUIRE(y.data != nullptr && matrices.data != nullptr, "Winograd output transform: null tensor");
+		mlTensor_t out = y;
+		if (y.dtype == DTYPE_FLOAT16)
+			launch_output<half_t>(stream, matrices, bias, ext, out, act);
+		else
+			launch_output<float>(stream, matrices, bias, ext, out, act);
+	}
+} /* extern "C" */
+
+MLHIP_ALSO_AS_CUDA(winograd_weight_transform)
+MLHIP_ALSO_AS_CUDA(winograd_input_transform)
+MLHIP_ALSO_AS_CUDA(winograd_output_transform)
