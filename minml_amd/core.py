@@ -218,6 +218,48 @@ def _require(cond, msg):
         raise ValueError(msg)
 
 
+class KernelTimer:
+    """Brackets every call of the named entry points with two events on the context's stream, so that the duration of each kernel is
+    measured where it runs; `summary()` returns {name: (launches, average seconds)}. Installed with set_kernel_timer()."""
+
+    def __init__(self, context):
+        self.context = context
+        self.records = {}
+
+    def call(self, name, function, *args):
+        start = Event(self.context)
+        function(*args)
+        end = Event(self.context)
+        self.records.setdefault(name, []).append((start, end))
+
+    def summary(self):
+        self.context.synchronize()
+        result = {}
+        for name, pairs in self.records.items():
+            total = sum(Event.getElapsedTime(s, e) for s, e in pairs)
+            result[name] = (len(pairs), total / len(pairs))
+            for s, e in pairs:
+                s.destroy()
+                e.destroy()
+        self.records = {}
+        return result
+
+
+_TIMER = None
+
+
+def set_kernel_timer(timer):
+    global _TIMER
+    _TIMER = timer
+
+
+def _launch(name, *args):
+    if _TIMER is None:
+        B.fn(name)(*args)
+    else:
+        _TIMER.call(name, B.fn(name), *args)
+
+
 def _same_dtype(*tensors):
     ts = [t for t in tensors if t is not None and not t.isEmpty()]
     return all(t.dtype == ts[0].dtype for t in ts)
@@ -241,7 +283,7 @@ def winogradWeightTransform(context, weights, matrices, invert=False):
     _require_winograd_supported(tile, weights.shape[1], weights.dtype)
     _require(_same_dtype(weights, matrices), "dtype mismatch")
     _require(matrices.shape == (36, weights.shape[0], weights.shape[3]), "matrices must be [36, Cout, Cin]")
-    B.fn("winograd_weight_transform")(context.handle, tile, weights.desc(), matrices.desc(), bool(invert))
+    _launch("winograd_weight_transform", context.handle, tile, weights.desc(), matrices.desc(), bool(invert))
 
 
 def winogradInputTransform(context, weight_shape, input, matrices):
@@ -250,7 +292,7 @@ def winogradInputTransform(context, weight_shape, input, matrices):
     _require(_same_dtype(input, matrices), "dtype mismatch")
     b, h, w, c = input.shape
     _require(matrices.shape == (36, b * ((h + 3) // 4) * ((w + 3) // 4), c), "matrices must be [36, tiles, C]")
-    B.fn("winograd_input_transform")(context.handle, tile, input.desc(), matrices.desc())
+    _launch("winograd_input_transform", context.handle, tile, input.desc(), matrices.desc())
 
 
 def winogradOutputTransform(context, weight_shape, matrices, output, bias, add, act):
@@ -261,7 +303,7 @@ def winogradOutputTransform(context, weight_shape, matrices, output, bias, add, 
     _require(matrices.shape == (36, b * ((h + 3) // 4) * ((w + 3) // 4), c), "matrices must be [36, tiles, C]")
     _require(bias is None or bias.isEmpty() or bias.volume() == c, "bias must be [C]")
     _require(add is None or add.isEmpty() or add.shape == output.shape, "add must have the output's shape")
-    B.fn("winograd_output_transform")(context.handle, tile, matrices.desc(), _desc(bias), _desc(add), output.desc(), act_of(act))
+    _launch("winograd_output_transform", context.handle, tile, matrices.desc(), _desc(bias), _desc(add), output.desc(), act_of(act))
 
 
 def _gemm_dims(opA, A, opB, Bm):
@@ -284,7 +326,7 @@ def gemm(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
         _require(A.dtype == B.DTYPE_INT8 and Bm.dtype == B.DTYPE_INT8 and alpha == 1.0 and beta == 0.0, "int8 product: int8 operands, alpha 1, beta 0")
     else:
         _require(_same_dtype(A, Bm, C) and C.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
-    B.fn("gemm_v2")(context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
+    _launch("gemm_v2", context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
 
 
 def gemmBatched(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
@@ -295,7 +337,7 @@ def gemmBatched(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
     _require(A.rank() == 2 or A.shape[0] == C.shape[0], "batch of A")
     _require(Bm.rank() == 2 or Bm.shape[0] == C.shape[0], "batch of B")
     _require(_same_dtype(A, Bm, C) and C.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
-    B.fn("gemm_batched_v2")(context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
+    _launch("gemm_batched_v2", context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
 
 
 def gemm_ex(context, D, alpha, opA, A, opB, Bm, beta, C, bias, act):
@@ -306,7 +348,7 @@ def gemm_ex(context, D, alpha, opA, A, opB, Bm, beta, C, bias, act):
     _require(_same_dtype(A, Bm, C, D, bias) and D.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
     _require(bias is None or bias.isEmpty() or bias.volume() == N, "bias must be [N]")
     c = C if (C is not None and not C.isEmpty()) else D
-    B.fn("gemm_ex")(context.handle, D.dtype, D.shape_desc(), D.ptr, alpha, opA.encode(), A.shape_desc(), A.ptr, opB.encode(), Bm.shape_desc(), Bm.ptr,
+    _launch("gemm_ex", context.handle, D.dtype, D.shape_desc(), D.ptr, alpha, opA.encode(), A.shape_desc(), A.ptr, opB.encode(), Bm.shape_desc(), Bm.ptr,
                     beta, c.shape_desc(), c.ptr, _ptr(bias), act_of(act))
 
 
@@ -317,7 +359,7 @@ def im2row(context, output, input, kernel_size, invert=False, padding=None):
     pad = None
     if padding is not None:
         pad = np.array([padding], _NP_OF[input.dtype])
-    B.fn("im2row")(context.handle, input.dtype, input.shape_desc(), output.ptr, input.ptr, kernel_size, bool(invert),
+    _launch("im2row", context.handle, input.dtype, input.shape_desc(), output.ptr, input.ptr, kernel_size, bool(invert),
                    None if pad is None else pad.ctypes.data_as(ctypes.c_void_p))
 
 
@@ -328,7 +370,7 @@ def convolutionImplicitGemmForward(context, input, weights, output, bias, add, a
     _require(output.shape[:3] == input.shape[:3], "stride 1, same padding")
     _require(_same_dtype(input, weights, output, bias, add) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
     _require(add is None or add.isEmpty() or add.shape == output.shape, "add must have the output's shape")
-    B.fn("convolution_implicit_gemm_forward")(context.handle, weights.dtype, input.shape_desc(), weights.shape_desc(), input.ptr, weights.ptr,
+    _launch("convolution_implicit_gemm_forward", context.handle, weights.dtype, input.shape_desc(), weights.shape_desc(), input.ptr, weights.ptr,
                                               output.ptr, _ptr(bias), _ptr(add), act_of(act))
 
 
@@ -357,7 +399,7 @@ def quantized_scale_shift_act(context, output, output_transform, input, scales, 
     _require(output.dtype in (B.DTYPE_INT8, B.DTYPE_FLOAT32, B.DTYPE_FLOAT16), "output must be int8, fp16 or fp32")
     _require(input.volume() == output.volume() and scales.volume() == output.lastDim() and bias.volume() == output.lastDim(), "shape mismatch")
     _require(ext is None or ext.isEmpty() or (ext.dtype == B.DTYPE_INT8 and ext.volume() == output.volume()), "ext must be int8 of the output's shape")
-    B.fn("quantized_scale_shift_act")(context.handle, output.dtype, output.shape_desc(), output.ptr, B.mlQuantizationData_t(*output_transform), input.ptr,
+    _launch("quantized_scale_shift_act", context.handle, output.dtype, output.shape_desc(), output.ptr, B.mlQuantizationData_t(*output_transform), input.ptr,
                                       scales.ptr, bias.ptr, act_of(act), _ptr(ext), B.mlQuantizationData_t(*ext_transform))
 
 
@@ -369,7 +411,7 @@ def quantizedConvForward(context, input, input_transform, weights, scales, bias,
     _require(output.dtype in (B.DTYPE_INT8, B.DTYPE_FLOAT32), "output must be int8 or fp32")
     _require(scales.volume() == weights.shape[0] and bias.volume() == weights.shape[0], "scales / bias must be [Cout]")
     _require(ext is None or ext.isEmpty() or (ext.dtype == B.DTYPE_INT8 and ext.shape == output.shape), "ext must be int8 of the output's shape")
-    B.fn("quantized_conv_forward")(context.handle, input.shape_desc(), weights.shape_desc(), input.ptr, B.mlQuantizationData_t(*input_transform),
+    _launch("quantized_conv_forward", context.handle, input.shape_desc(), weights.shape_desc(), input.ptr, B.mlQuantizationData_t(*input_transform),
                                    weights.ptr, scales.ptr, bias.ptr, output.dtype, output.ptr, B.mlQuantizationData_t(*output_transform), _ptr(ext),
                                    B.mlQuantizationData_t(*ext_transform), act_of(act))
 

@@ -211,7 +211,6 @@ extern "C"
 	void hip_convolution_implicit_gemm_forward(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, mlShape_t weights_shape,
 			const void *input, const void *weights, void *output, const void *bias, const void *add, mlActivationType_t act)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(input_shape.rank == 4 && weights_shape.rank == 4, "convolution: input must be [B,H,W,Cin] and weights [Cout,k,k,Cin]");
 		MLHIP_REQUIRE(input_shape.dim[3] == weights_shape.dim[3], "convolution: input and weights disagree on the number of input filters");
 		MLHIP_REQUIRE(dtype == DTYPE_FLOAT16 || dtype == DTYPE_FLOAT32, "convolution: unsupported data type");
@@ -219,15 +218,14 @@ extern "C"
 			return;
 		MLHIP_REQUIRE(input != nullptr && weights != nullptr && output != nullptr, "convolution: null tensor");
 		if (dtype == DTYPE_FLOAT16)
-			conv_forward<half_t>(stream, dtype, input_shape, weights_shape, input, weights, output, bias, add, act);
+			conv_forward<half_t>(stream_of(context), dtype, input_shape, weights_shape, input, weights, output, bias, add, act);
 		else
-			conv_forward<float>(stream, dtype, input_shape, weights_shape, input, weights, output, bias, add, act);
+			conv_forward<float>(stream_of(context), dtype, input_shape, weights_shape, input, weights, output, bias, add, act);
 	}
 
 	void hip_im2row(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, void *output, const void *input, int kernel_size, bool invert,
 			const void *padding)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(input_shape.rank == 4, "im2row: input must be [B,H,W,C]");
 		MLHIP_REQUIRE(kernel_size >= 1, "im2row: kernel size must be positive");
 		const int esize = size_of(dtype);
@@ -247,7 +245,7 @@ extern "C"
 		{
 			uint4_t p;
 			std::memcpy(&p, pad, 16);
-			launch_im2row<uint4_t>(stream, input, output, batch, height, width, static_cast<int>(c_bytes / 16), kernel_size, invert, p);
+			launch_im2row<uint4_t>(stream_of(context), input, output, batch, height, width, static_cast<int>(c_bytes / 16), kernel_size, invert, p);
 		}
 		else
 			switch (esize)
@@ -256,28 +254,28 @@ extern "C"
 				{
 					uint8_t p;
 					std::memcpy(&p, pad, 1);
-					launch_im2row<uint8_t>(stream, input, output, batch, height, width, channels, kernel_size, invert, p);
+					launch_im2row<uint8_t>(stream_of(context), input, output, batch, height, width, channels, kernel_size, invert, p);
 					break;
 				}
 				case 2:
 				{
 					uint16_t p;
 					std::memcpy(&p, pad, 2);
-					launch_im2row<uint16_t>(stream, input, output, batch, height, width, channels, kernel_size, invert, p);
+					launch_im2row<uint16_t>(stream_of(context), input, output, batch, height, width, channels, kernel_size, invert, p);
 					break;
 				}
 				case 4:
 				{
 					uint32_t p;
 					std::memcpy(&p, pad, 4);
-					launch_im2row<uint32_t>(stream, input, output, batch, height, width, channels, kernel_size, invert, p);
+					launch_im2row<uint32_t>(stream_of(context), input, output, batch, height, width, channels, kernel_size, invert, p);
 					break;
 				}
 				default:
 				{
 					uint64_t p;
 					std::memcpy(&p, pad, 8);
-					launch_im2row<uint64_t>(stream, input, output, batch, height, width, channels, kernel_size, invert, p);
+					launch_im2row<uint64_t>(stream_of(context), input, output, batch, height, width, channels, kernel_size, invert, p);
 					break;
 				}
 			}

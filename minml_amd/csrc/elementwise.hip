@@ -158,7 +158,6 @@ extern "C"
 
 	void hip_add_bias_act(mlContext_t context, float alpha, const mlTensor_t x, const mlTensor_t b, float beta, mlTensor_t y, mlActivationType_t act)
 	{
-		hipStream_t stream = stream_of(context);
 		if (volume(x) == 0)
 			return;
 		MLHIP_REQUIRE(x.dtype == y.dtype && volume(x) == volume(y), "add_bias_act: x and y must have one shape and data type");
@@ -169,10 +168,10 @@ extern "C"
 		switch (x.dtype)
 		{
 			case DTYPE_FLOAT16:
-				launch_add_bias_act<half_t>(stream, alpha, x, b, beta, out, act);
+				launch_add_bias_act<half_t>(stream_of(context), alpha, x, b, beta, out, act);
 				break;
 			case DTYPE_FLOAT32:
-				launch_add_bias_act<float>(stream, alpha, x, b, beta, out, act);
+				launch_add_bias_act<float>(stream_of(context), alpha, x, b, beta, out, act);
 				break;
 			default:
 				fail_logic("HIP backend: add_bias_act: unsupported data type");
@@ -211,17 +210,16 @@ extern "C"
 	void hip_add_tensors(mlContext_t context, float alpha1, const mlTensor_t x1, float alpha2, const mlTensor_t x2, float alpha3, const mlTensor_t x3,
 			float beta, mlTensor_t y)
 	{
-		hipStream_t stream = stream_of(context);
 		if (volume(y) == 0 || y.data == nullptr)
 			return;
 		mlTensor_t out = y;
 		switch (y.dtype)
 		{
 			case DTYPE_FLOAT16:
-				launch_axpy3<half_t>(stream, alpha1, x1, alpha2, x2, alpha3, x3, beta, out);
+				launch_axpy3<half_t>(stream_of(context), alpha1, x1, alpha2, x2, alpha3, x3, beta, out);
 				break;
 			case DTYPE_FLOAT32:
-				launch_axpy3<float>(stream, alpha1, x1, alpha2, x2, alpha3, x3, beta, out);
+				launch_axpy3<float>(stream_of(context), alpha1, x1, alpha2, x2, alpha3, x3, beta, out);
 				break;
 			default:
 				fail_logic("HIP backend: add_tensors: unsupported data type");
@@ -246,13 +244,12 @@ extern "C"
 				hip_memcpy_within_device(context, dst, 0, src, 0, static_cast<size_t>(elements) * size_of(dst_dtype));
 			return;
 		}
-		hipStream_t stream = stream_of(context);
 		const size_t n = static_cast<size_t>(elements);
 		if (src_dtype == DTYPE_FLOAT32 && dst_dtype == DTYPE_FLOAT16)
-			hipLaunchKernelGGL((kernel_convert<half_t, float>), dim3(grid_for(n)), dim3(256), 0, stream, reinterpret_cast<half_t*>(dst),
+			hipLaunchKernelGGL((kernel_convert<half_t, float>), dim3(grid_for(n)), dim3(256), 0, stream_of(context), reinterpret_cast<half_t*>(dst),
 					reinterpret_cast<const float*>(src), n);
 		else if (src_dtype == DTYPE_FLOAT16 && dst_dtype == DTYPE_FLOAT32)
-			hipLaunchKernelGGL((kernel_convert<float, half_t>), dim3(grid_for(n)), dim3(256), 0, stream, reinterpret_cast<float*>(dst),
+			hipLaunchKernelGGL((kernel_convert<float, half_t>), dim3(grid_for(n)), dim3(256), 0, stream_of(context), reinterpret_cast<float*>(dst),
 					reinterpret_cast<const half_t*>(src), n);
 		else
 			fail_logic("unsupported conversion");
@@ -260,7 +257,6 @@ extern "C"
 	}
 	void hip_unpack_input(mlContext_t context, mlShape_t shape, mlDataType_t dst_dtype, void *dst, const void *src)
 	{
-		hipStream_t stream = stream_of(context);
 		if (volume(shape) == 0)
 			return;
 		MLHIP_REQUIRE(dst != nullptr && src != nullptr, "unpack_input: null pointer");
@@ -271,22 +267,22 @@ extern "C"
 		switch (dst_dtype)
 		{
 			case DTYPE_FLOAT16:
-				hipLaunchKernelGGL(kernel_unpack_input<half_t>, grid, block, 0, stream, reinterpret_cast<half_t*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<half_t>, grid, block, 0, stream_of(context), reinterpret_cast<half_t*>(dst), in, first, last);
 				break;
 			case DTYPE_FLOAT32:
-				hipLaunchKernelGGL(kernel_unpack_input<float>, grid, block, 0, stream, reinterpret_cast<float*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<float>, grid, block, 0, stream_of(context), reinterpret_cast<float*>(dst), in, first, last);
 				break;
 			case DTYPE_UINT8:
-				hipLaunchKernelGGL(kernel_unpack_input<uint8_t>, grid, block, 0, stream, reinterpret_cast<uint8_t*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<uint8_t>, grid, block, 0, stream_of(context), reinterpret_cast<uint8_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT8:
-				hipLaunchKernelGGL(kernel_unpack_input<int8_t>, grid, block, 0, stream, reinterpret_cast<int8_t*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<int8_t>, grid, block, 0, stream_of(context), reinterpret_cast<int8_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT16:
-				hipLaunchKernelGGL(kernel_unpack_input<int16_t>, grid, block, 0, stream, reinterpret_cast<int16_t*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<int16_t>, grid, block, 0, stream_of(context), reinterpret_cast<int16_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT32:
-				hipLaunchKernelGGL(kernel_unpack_input<int32_t>, grid, block, 0, stream, reinterpret_cast<int32_t*>(dst), in, first, last);
+				hipLaunchKernelGGL(kernel_unpack_input<int32_t>, grid, block, 0, stream_of(context), reinterpret_cast<int32_t*>(dst), in, first, last);
 				break;
 			default:
 				fail_logic("HIP backend: unpack_input: unsupported destination type");

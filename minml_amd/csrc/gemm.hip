@@ -222,6 +222,16 @@ namespace mlhip
 	}
 }
 
+namespace
+{
+	void run_gemm(mlContext_t context, const mlhip::GemmArgs &g)
+	{
+		if (g.M == 0 || g.N == 0 || g.batch == 0)
+			return; /* nothing to compute: no context needed */
+		mlhip::launch_gemm(mlhip::stream_of(context), g);
+	}
+}
+
 extern "C"
 {
 	using namespace mlhip;
@@ -236,7 +246,7 @@ extern "C"
 		g.D = C;
 		g.alpha = alpha;
 		g.beta = beta;
-		launch_gemm(stream_of(context), g);
+		run_gemm(context, g);
 	}
 	void hip_gemm_batched(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
 			const void *B, char opA, char opB, float alpha, float beta)
@@ -248,7 +258,7 @@ extern "C"
 		g.D = C;
 		g.alpha = alpha;
 		g.beta = beta;
-		launch_gemm(stream_of(context), g);
+		run_gemm(context, g);
 	}
 	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
 	{
@@ -284,7 +294,7 @@ extern "C"
 		g.beta = beta;
 		g.bias = bias;
 		g.act = act;
-		launch_gemm(stream_of(context), g);
+		run_gemm(context, g);
 	}
 } /* extern "C" */
 

@@ -208,7 +208,6 @@ extern "C"
 	void hip_quantized_scale_shift_act(mlContext_t context, mlDataType_t dtype, mlShape_t shape, void *output, mlQuantizationData_t output_qd,
 			const void *input, const void *scales, const void *bias, mlActivationType_t act, const void *ext, mlQuantizationData_t ext_qd)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(shape.rank >= 1, "quantized_scale_shift_act: empty shape");
 		if (volume(shape) == 0)
 			return;
@@ -216,13 +215,13 @@ extern "C"
 		switch (dtype)
 		{
 			case DTYPE_INT8:
-				launch_scale_shift_act<int8_t>(stream, shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
+				launch_scale_shift_act<int8_t>(stream_of(context), shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
 				break;
 			case DTYPE_FLOAT32:
-				launch_scale_shift_act<float>(stream, shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
+				launch_scale_shift_act<float>(stream_of(context), shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
 				break;
 			case DTYPE_FLOAT16:
-				launch_scale_shift_act<half_t>(stream, shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
+				launch_scale_shift_act<half_t>(stream_of(context), shape, output, output_qd, input, scales, bias, act, ext, ext_qd);
 				break;
 			default:
 				fail_logic("HIP backend: quantized_scale_shift_act: output must be INT8, FLOAT16 or FLOAT32");
@@ -233,7 +232,6 @@ extern "C"
 			mlQuantizationData_t input_qd, const void *weights, const void *scales, const void *bias, mlDataType_t output_dtype, void *output,
 			mlQuantizationData_t output_qd, const void *ext, mlQuantizationData_t ext_qd, mlActivationType_t act)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(input_shape.rank == 4 && weights_shape.rank == 4, "quantized convolution: input must be [B,H,W,Cin] and weights [Cout,k,k,Cin]");
 		MLHIP_REQUIRE(input_shape.dim[3] == weights_shape.dim[3], "quantized convolution: input and weights disagree on the number of input filters");
 		if (volume(input_shape) == 0 || weights_shape.dim[0] == 0)
@@ -243,10 +241,10 @@ extern "C"
 		switch (output_dtype)
 		{
 			case DTYPE_INT8:
-				launch_quantized_conv<int8_t>(stream, input_shape, weights_shape, input, input_qd, weights, scales, bias, output, output_qd, ext, ext_qd, act);
+				launch_quantized_conv<int8_t>(stream_of(context), input_shape, weights_shape, input, input_qd, weights, scales, bias, output, output_qd, ext, ext_qd, act);
 				break;
 			case DTYPE_FLOAT32:
-				launch_quantized_conv<float>(stream, input_shape, weights_shape, input, input_qd, weights, scales, bias, output, output_qd, ext, ext_qd, act);
+				launch_quantized_conv<float>(stream_of(context), input_shape, weights_shape, input, input_qd, weights, scales, bias, output, output_qd, ext, ext_qd, act);
 				break;
 			default:
 				fail_logic("HIP backend: quantized convolution: output must be INT8 or FLOAT32");

@@ -414,7 +414,6 @@ extern "C"
 
 	void hip_winograd_weight_transform(mlContext_t context, int tile_size, const mlTensor_t w, mlTensor_t matrices, bool invert)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(w.rank == 4 && w.dim[1] == w.dim[2], "Winograd weights must be [Cout, k, k, Cin] with a square kernel");
 		require_supported(tile_size, matrices, w.dtype);
 		MLHIP_REQUIRE(w.dim[1] == 3, "Winograd weight transform: weight kernel size does not match the matrices");
@@ -428,16 +427,15 @@ extern "C"
 		const dim3 block(256);
 		const dim3 grid(grid_for(threads));
 		if (w.dtype == DTYPE_FLOAT16)
-			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<half_t>, grid, block, 0, stream, ptr<const half_t>(w), ptr<half_t>(matrices), w.dim[0],
+			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<half_t>, grid, block, 0, stream_of(context), ptr<const half_t>(w), ptr<half_t>(matrices), w.dim[0],
 					w.dim[3], invert);
 		else
-			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<float>, grid, block, 0, stream, ptr<const float>(w), ptr<float>(matrices), w.dim[0],
+			hipLaunchKernelGGL(kernel_weight_transform_4x4_3x3<float>, grid, block, 0, stream_of(context), ptr<const float>(w), ptr<float>(matrices), w.dim[0],
 					w.dim[3], invert);
 		MLHIP_CHECK(hipGetLastError());
 	}
 	void hip_winograd_input_transform(mlContext_t context, int tile_size, const mlTensor_t x, mlTensor_t matrices)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(x.rank == 4, "Winograd input transform: input must be [B, H, W, C]");
 		require_supported(tile_size, matrices, x.dtype);
 		MLHIP_REQUIRE(matrices.dtype == x.dtype, "Winograd input transform: dtype mismatch");
@@ -449,14 +447,13 @@ extern "C"
 		MLHIP_REQUIRE(x.data != nullptr && matrices.data != nullptr, "Winograd input transform: null tensor");
 		mlTensor_t m = matrices;
 		if (x.dtype == DTYPE_FLOAT16)
-			launch_input<half_t>(stream, x, m);
+			launch_input<half_t>(stream_of(context), x, m);
 		else
-			launch_input<float>(stream, x, m);
+			launch_input<float>(stream_of(context), x, m);
 	}
 	void hip_winograd_output_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
 			mlTensor_t y, mlActivationType_t act)
 	{
-		hipStream_t stream = stream_of(context);
 		MLHIP_REQUIRE(y.rank == 4, "Winograd output transform: output must be [B, H, W, C]");
 		require_supported(tile_size, matrices, y.dtype);
 		MLHIP_REQUIRE(matrices.dtype == y.dtype, "Winograd output transform: dtype mismatch");
@@ -472,9 +469,9 @@ extern "C"
 		MLHIP_REQUIRE(y.data != nullptr && matrices.data != nullptr, "Winograd output transform: null tensor");
 		mlTensor_t out = y;
 		if (y.dtype == DTYPE_FLOAT16)
-			launch_output<half_t>(stream, matrices, bias, ext, out, act);
+			launch_output<half_t>(stream_of(context), matrices, bias, ext, out, act);
 		else
-			launch_output<float>(stream, matrices, bias, ext, out, act);
+			launch_output<float>(stream_of(context), matrices, bias, ext, out, act);
 	}
 } /* extern "C" */
 

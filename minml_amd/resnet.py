@@ -16,6 +16,10 @@ from . import core as ml
 from .conv2d import Conv2D
 
 
+# positions per sub-batch pushed through the whole network at once, by storage type (measured choice; see ResNet docstring)
+DEFAULT_CHUNK = {"float16": 1024, "float32": 256}
+
+
 def he_normal_weights(rng, shape):
     """He-normal: sigma = sqrt(2 / fan_in), fan_in = k*k*Cin."""
     fan_in = shape[1] * shape[2] * shape[3]

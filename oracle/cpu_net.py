@@ -1,0 +1,66 @@
+"""CPU execution of the synthetic residual network, layer by layer, for checking and for the CPU-baseline timing.
+
+TEST INFRASTRUCTURE ONLY (see oracle/__init__.py). Two engines with one interface:
+  * engine="oracle":     this repository's C restatement (oracle.c), optionally multi-threaded;
+  * engine="reference":  the reference's own CPU backend compiled into oracle/_ref (single-threaded, as the reference runs it:
+                         its GEMM has no threading and the OpenMP pragmas of its input / output transforms are commented out,
+                         src/backend/cpu/winograd/winograd_runtime.cpp:121,133,180,198).
+Both run every 3x3 convolution as Winograd F(4x4,3x3): weight transform (cached) -> input transform -> 36 batched GEMMs ('n','t')
+-> output transform with bias, residual and ReLU; the 1x1 head is gemm_ex on the [B*H*W, C] view — the call sequence of
+src/layers/Conv2D.cpp:329-378.
+"""
+import time
+
+import numpy as np
+
+import oracle as O
+
+
+class CpuResNet:
+    def __init__(self, params_storage, blocks, engine="oracle"):
+        """params_storage: list of (weights, bias) already in the storage type (float32 arrays or uint16 fp16 bit patterns)."""
+        self.blocks = blocks
+        self.params = params_storage
+        self.engine = engine
+        self.ref = O.reference() if engine == "reference" else None
+        if engine == "reference" and self.ref is None:
+            raise RuntimeError("oracle/_ref is not built")
+        e = self.ref if self.ref is not None else O
+        self.transformed = [e.winograd_weight_transform(w) if w.shape[1] == 3 else None for (w, _) in params_storage]
+
+    def _conv3x3(self, idx, x, add, act):
+        w, b = self.params[idx]
+        e = self.ref if self.ref is not None else O
+        v = e.winograd_input_transform(x)
+        if self.ref is not None:
+            m = self.ref.gemm_batched(v, self.transformed[idx])
+        else:
+            m = O.gemm(v, self.transformed[idx])
+        shape = x.shape[:3] + (w.shape[0],)
+        return e.winograd_output_transform(m, shape, b, add, act)
+
+    def forward(self, x, return_trunk=False):
+        a = self._conv3x3(0, x, None, O.RELU)
+        for blk in range(self.blocks):
+            t = self._conv3x3(1 + 2 * blk, a, None, O.RELU)
+            a = self._conv3x3(2 + 2 * blk, t, a, O.RELU)
+        w, b = self.params[-1]
+        rows = a.shape[0] * a.shape[1] * a.shape[2]
+        am = a.reshape(rows, a.shape[3])
+        wm = w.reshape(w.shape[0], -1)
+        if self.ref is not None:
+            head = self.ref.gemm_ex(am, wm, bias=b, act=O.LINEAR)
+        else:
+            head = O.gemm(am, wm, bias=b, act=O.LINEAR)
+        head = head.reshape(a.shape[:3] + (w.shape[0],))
+        return (head, a) if return_trunk else head
+
+    def timed_forward(self, x, repeats=1):
+        """Seconds per forward pass (best of `repeats`, after the weight transforms that __init__ already did)."""
+        best = None
+        for _ in range(repeats):
+            t0 = time.perf_counter()
+            self.forward(x)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+        return best

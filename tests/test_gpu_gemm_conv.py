@@ -1,0 +1,225 @@
+"""GEMM entry points and fused convolution on the GPU against the CPU oracle, through the C-ABI.
+
+Tolerances (max-abs relative error per result tensor, as stated for this path): fp32 1e-4, fp16 1e-2. The oracle accumulates like the
+reference (sequential fused multiply-adds, K split at 1024 with a rounded intermediate store); the MFMA kernels accumulate the whole K
+extent in fp32, so results agree to rounding, not bit for bit. im2row is byte movement and is compared exactly."""
+import numpy as np
+import pytest
+
+import oracle as O
+from minml_amd import core as ml
+from util import TOL, max_abs_rel, mean_abs_diff, mismatches, random_tensor, init_for_test, storage
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("ops", ["nn", "nt", "tn", "tt"])
+def test_gemm_all_ops(ctx, dtype, ops):
+    """test/backend/test_gemms.cpp:178-374: 23 x 45 x 67, alpha = 1.1, beta = 0.1, mean-abs-diff <= 1e-4 (fp16: 1e-2)."""
+    M, N, K = 23, 45, 67
+    A = storage(init_for_test((M, K) if ops[0] == "n" else (K, M), 0.0), dtype)
+    Bm = storage(init_for_test((K, N) if ops[1] == "n" else (N, K), 1.0), dtype)
+    C = storage(init_for_test((M, N), 2.0), dtype)
+    dC = ml.toDevice(ctx, C)
+    ml.gemm(ctx, ops[0], ops[1], dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.1, 0.1)
+    want = O.gemm(A, Bm, ops[0], ops[1], alpha=1.1, beta=0.1, C=C)
+    assert mean_abs_diff(dC.copyToHost(ctx), want) <= (1e-4 if dtype == "float32" else 1e-2)
+    assert max_abs_rel(dC.copyToHost(ctx), want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("shape", [(36, 48, 21, 35), (5, 77, 33, 40), (3, 300, 256, 256), (2, 130, 70, 264), (36, 16 * 8, 256, 32), (1, 1, 1, 8),
+                                   (2, 129, 129, 1032)])
+def test_gemm_batched_nt(ctx, dtype, shape):
+    """The Winograd product M[i] = V[i] * U[i]^T: ragged M and N, K that is no multiple of the pipeline step, K > 1024."""
+    bt, M, N, K = shape
+    rng = np.random.default_rng(sum(shape))
+    A = random_tensor(rng, (bt, M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (bt, N, K), dtype, 0.5)
+    dC = ml.Tensor((bt, M, N), dtype)
+    dC.setall(ctx, float("nan"))  # beta = 0 must not read C (the reference's workspace is uninitialised)
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.0, 0.0)
+    got = dC.copyToHost(ctx)
+    assert np.isfinite(O.as_float(got)).all()
+    assert max_abs_rel(got, O.gemm(A, Bm)) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_gemm_batched_broadcast_and_beta(ctx, dtype):
+    rng = np.random.default_rng(5)
+    A = random_tensor(rng, (4, 50, 24), dtype)
+    Bm = random_tensor(rng, (30, 24), dtype)  # rank 2: broadcast (src/backend/cpu/gemm/gemm.cpp:18-29)
+    C = random_tensor(rng, (4, 50, 30), dtype)
+    dC = ml.toDevice(ctx, C)
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 0.5, 2.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm, alpha=0.5, beta=2.0, C=C)) <= TOL[dtype]
+    # transposed batched forms (used by the reference's training path) run on the generic kernel
+    At = random_tensor(rng, (3, 24, 50), dtype)
+    Bn = random_tensor(rng, (3, 24, 30), dtype)
+    dC = ml.Tensor((3, 50, 30), dtype)
+    ml.gemmBatched(ctx, "t", "n", dC, ml.toDevice(ctx, At), ml.toDevice(ctx, Bn), 1.0, 0.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(At, Bn, "t", "n")) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("act", ["linear", "relu", "sigmoid", "tanh"])
+def test_gemm_ex_epilogue(ctx, dtype, act):
+    """D = act(alpha A B^T + bias + beta C), C distinct from D (test/backend/test_gemms.cpp gemm_ex, src/backend/cpu/gemm/gemm.cpp:66-83)."""
+    rng = np.random.default_rng(6)
+    for (M, N, K) in ((123, 45, 72), (23, 45, 67), (500, 1, 256), (64, 128, 2304), (257, 136, 40)):
+        A = random_tensor(rng, (M, K), dtype, 0.3)
+        Bm = random_tensor(rng, (N, K), dtype, 0.3)
+        C = random_tensor(rng, (M, N), dtype)
+        bias = random_tensor(rng, (N,), dtype)
+        dD = ml.Tensor((M, N), dtype)
+        ml.gemm_ex(ctx, dD, 1.1, "n", ml.toDevice(ctx, A), "t", ml.toDevice(ctx, Bm), 0.1, ml.toDevice(ctx, C), ml.toDevice(ctx, bias), act)
+        want = O.gemm(A, Bm, alpha=1.1, beta=0.1, C=C, bias=bias, act=ml.act_of(act))
+        assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype]
+        # in place (C is D) and without bias
+        dD = ml.toDevice(ctx, C)
+        ml.gemm_ex(ctx, dD, 1.0, "n", ml.toDevice(ctx, A), "t", ml.toDevice(ctx, Bm), 1.0, dD, None, act)
+        want = O.gemm(A, Bm, alpha=1.0, beta=1.0, C=C, act=ml.act_of(act))
+        assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("tag,dtype", [("f32", "float32"), ("f16", "float16")])
+def test_reference_fixtures(ctx, golden, tag, dtype):
+    g = golden
+    dD = ml.Tensor((23, 45), dtype)
+    ml.gemm_ex(ctx, dD, 1.1, "n", ml.toDevice(ctx, g["ge_a_" + tag]), "t", ml.toDevice(ctx, g["ge_b_" + tag]), 0.1, ml.toDevice(ctx, g["ge_c_" + tag]),
+               ml.toDevice(ctx, g["ge_bias_" + tag]), "relu")
+    assert max_abs_rel(dD.copyToHost(ctx), g["ge_d_" + tag]) <= TOL[dtype]
+    dD = ml.Tensor((9, 7), dtype)
+    ml.gemm_ex(ctx, dD, 1.0, "n", ml.toDevice(ctx, g["gk_a_" + tag]), "t", ml.toDevice(ctx, g["gk_b_" + tag]), 0.0, None, None, "linear")
+    assert max_abs_rel(dD.copyToHost(ctx), g["gk_d_" + tag]) <= TOL[dtype]
+    rows = ml.Tensor((2 * 7 * 6, 25 * 8), dtype)
+    ml.im2row(ctx, rows, ml.toDevice(ctx, g["cv_x_" + tag]), 5)
+    assert mismatches(rows.copyToHost(ctx), g["cv_rows_" + tag]) == 0
+    dy = ml.Tensor((2, 7, 6, 12), dtype)
+    ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, g["cv_x_" + tag]), ml.toDevice(ctx, g["cv_w_" + tag]), dy, ml.toDevice(ctx, g["cv_bias_" + tag]),
+                                      ml.toDevice(ctx, g["cv_add_" + tag]), "relu")
+    assert max_abs_rel(dy.copyToHost(ctx), g["cv_y_" + tag]) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16", "int8"])
+@pytest.mark.parametrize("shape,k", [((2, 7, 6, 16), 5), ((3, 5, 4, 3), 3), ((1, 19, 19, 8), 5), ((2, 6, 5, 7), 3), ((4, 12, 14, 32), 3)])
+def test_im2row_exact(ctx, dtype, shape, k):
+    """test/backend/test_gemm_conv.cpp:68-150: EXPECT_EQ(diff, 0)."""
+    rng = np.random.default_rng(k + shape[3])
+    x = rng.integers(-128, 128, shape).astype(np.int8) if dtype == "int8" else random_tensor(rng, shape, dtype)
+    rows = ml.Tensor((shape[0] * shape[1] * shape[2], k * k * shape[3]), dtype)
+    ml.im2row(ctx, rows, ml.toDevice(ctx, x), k)
+    assert mismatches(rows.copyToHost(ctx), O.im2row(x, k)) == 0
+    if dtype == "int8":  # padding with a zero point: same as shifting the data, gathering with zeros, shifting back
+        ml.im2row(ctx, rows, ml.toDevice(ctx, x), k, False, -37)
+        shifted = (x.astype(np.int16) + 37)
+        want = O.im2row(shifted.astype(np.float32), k).astype(np.int16) - 37
+        assert mismatches(rows.copyToHost(ctx), want.astype(np.int8)) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("shape,cout,k", [((2, 7, 6, 16), 24, 5), ((2, 9, 9, 32), 40, 3), ((3, 5, 7, 24), 8, 1), ((2, 6, 5, 7), 9, 3),
+                                          ((1, 19, 19, 64), 64, 5), ((2, 19, 19, 64), 64, 1), ((1, 19, 19, 128), 128, 3), ((2, 15, 15, 256), 1, 1)])
+def test_fused_convolution(ctx, dtype, shape, cout, k):
+    """hip_convolution_implicit_gemm_forward and the reference's explicit sequence (im2row + gemm_ex) against explicit_gemm_forward of the
+    oracle, with the fused bias + residual + ReLU epilogue (test/backend/test_conv2D.cpp:204-248,332-368,437-578)."""
+    rng = np.random.default_rng(cout + k)
+    b, h, w, cin = shape
+    x = random_tensor(rng, shape, dtype)
+    wt = random_tensor(rng, (cout, k, k, cin), dtype, (2.0 / (k * k * cin)) ** 0.5)
+    bias = random_tensor(rng, (cout,), dtype)
+    add = random_tensor(rng, (b, h, w, cout), dtype)
+    dx, dw, db, da = ml.toDevice(ctx, x), ml.toDevice(ctx, wt), ml.toDevice(ctx, bias), ml.toDevice(ctx, add)
+    want = O.conv2d_forward(x, wt, bias, add, O.RELU)
+    dy = ml.Tensor((b, h, w, cout), dtype)
+    ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, db, da, "relu")
+    assert max_abs_rel(dy.copyToHost(ctx), want) <= TOL[dtype]
+    ws = ml.Tensor((max(1, b * h * w * k * k * cin),), dtype)
+    dy2 = ml.Tensor((b, h, w, cout), dtype)
+    ml.explicit_gemm_forward(ctx, dx, dy2, dw, db, ws, "relu", da)
+    assert max_abs_rel(dy2.copyToHost(ctx), want) <= TOL[dtype]
+    # no bias, no residual, linear
+    ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, None, None, "linear")
+    assert max_abs_rel(dy.copyToHost(ctx), O.conv2d_forward(x, wt)) <= TOL[dtype]
+
+
+def test_conv_sweep_config4_shapes(ctx):
+    """19x19 boards, fp16, channel widths {64,128,256,384}, kernels 1 / 3 / 5 with bias + ReLU + residual, at a batch the oracle finishes."""
+    rng = np.random.default_rng(44)
+    for c in (64, 128, 256, 384):
+        for k in (1, 3, 5):
+            x = random_tensor(rng, (2, 19, 19, c), "float16")
+            wt = random_tensor(rng, (c, k, k, c), "float16", (2.0 / (k * k * c)) ** 0.5)
+            bias = random_tensor(rng, (c,), "float16", 0.01)
+            add = random_tensor(rng, (2, 19, 19, c), "float16")
+            dy = ml.Tensor((2, 19, 19, c), "float16")
+            ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), ml.toDevice(ctx, wt), dy, ml.toDevice(ctx, bias), ml.toDevice(ctx, add), "relu")
+            assert max_abs_rel(dy.copyToHost(ctx), O.conv2d_forward(x, wt, bias, add, O.RELU)) <= 1e-2
+
+
+def test_convolution_linearity_at_full_size(ctx):
+    """Size-independent property at config 4's full size (B = 512, 19x19, 128 channels, 5x5, fp32 so that sums are comparable):
+    conv(x1 + x2) = conv(x1) + conv(x2) to rounding, and shifting the batch shifts the output."""
+    rng = np.random.default_rng(45)
+    shape = (512, 19, 19, 128)
+    x1 = (rng.integers(-4, 5, shape)).astype(np.float32)  # small integers: products and sums are exact in fp32
+    x2 = (rng.integers(-4, 5, shape)).astype(np.float32)
+    wt = rng.integers(-2, 3, (128, 5, 5, 128)).astype(np.float32)
+    dw = ml.toDevice(ctx, wt)
+    outs = []
+    for x in (x1, x2, x1 + x2):
+        dy = ml.Tensor(shape[:3] + (128,), "float32")
+        ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), dw, dy, None, None, "linear")
+        outs.append(dy.copyToHost(ctx))
+    assert np.array_equal(outs[0] + outs[1], outs[2])
+    sample = O.conv2d_forward(x1[100:101], wt)
+    assert np.array_equal(outs[0][100:101], sample)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_elementwise_neighbours(ctx, dtype):
+    rng = np.random.default_rng(7)
+    x = random_tensor(rng, (6, 5, 7, 12), dtype)
+    b = random_tensor(rng, (12,), dtype)
+    y0 = random_tensor(rng, (6, 5, 7, 12), dtype)
+    for act in ("linear", "relu", "sigmoid", "tanh", "leaky_relu", "exp"):
+        dy = ml.Tensor(x.shape, dtype)
+        ml.addBiasAct(ctx, 1.0, ml.toDevice(ctx, x), ml.toDevice(ctx, b), 0.0, dy, act)
+        assert max_abs_rel(dy.copyToHost(ctx), O.add_bias_act(x, b, ml.act_of(act))) <= TOL[dtype]
+        dy = ml.toDevice(ctx, y0)
+        ml.activationForward(ctx, 1.0, ml.toDevice(ctx, x), 0.0, dy, act)
+        assert max_abs_rel(dy.copyToHost(ctx), O.add_bias_act(x, None, ml.act_of(act))) <= TOL[dtype]
+    # y = act(x + b) * alpha + beta * y
+    dy = ml.toDevice(ctx, y0)
+    ml.addBiasAct(ctx, 0.5, ml.toDevice(ctx, x), ml.toDevice(ctx, b), 2.0, dy, "relu")
+    want = 0.5 * O.as_float(O.add_bias_act(x, b, O.RELU)).astype(np.float64) + 2.0 * O.as_float(y0)
+    assert np.abs(O.as_float(dy.copyToHost(ctx)) - want).max() / np.abs(want).max() <= TOL[dtype]
+    # odd last dimension (scalar path)
+    xo = random_tensor(rng, (9, 7), dtype)
+    bo = random_tensor(rng, (7,), dtype)
+    dy = ml.Tensor((9, 7), dtype)
+    ml.addBiasAct(ctx, 1.0, ml.toDevice(ctx, xo), ml.toDevice(ctx, bo), 0.0, dy, "relu")
+    assert mismatches(dy.copyToHost(ctx), O.add_bias_act(xo, bo, O.RELU)) == 0
+    # weighted sum and scaling
+    dy = ml.toDevice(ctx, y0)
+    ml.addTensors(ctx, 0.5, ml.toDevice(ctx, x), -2.0, ml.toDevice(ctx, x), 0.0, None, 0.25, dy)
+    assert max_abs_rel(dy.copyToHost(ctx), O.add_tensors(y0, 0.5, x, -2.0, x, 0.0, None, 0.25)) <= TOL[dtype]
+
+
+def test_convert_and_unpack(ctx, golden):
+    g = golden
+    src = g["cvt_src"]
+    dst = ml.Tensor(src.shape, "float16")
+    ml.convertType(ctx, dst, ml.toDevice(ctx, src))
+    got = dst.copyToHost(ctx)
+    assert mismatches(got, O.to_half(src)[...]) <= 1  # 65519.9: infinity by the reference's scalar rule, largest finite half by its vector rule
+    finite = np.abs(src) < 65504.0
+    assert mismatches(got[finite], g["cvt_f16"][finite]) == 0
+    back = ml.Tensor(src.shape, "float32")
+    ml.convertType(ctx, back, dst)
+    assert np.array_equal(back.copyToHost(ctx)[finite], O.from_half(got)[finite])
+    for code, key in ((O.FLOAT32, "up_f32"), (O.FLOAT16, "up_f16")):
+        d = ml.Tensor((3, 5, 40), code)
+        ml.unpackInput(ctx, d, ml.toDevice(ctx, g["up_packed"].view(np.int32), "int32"))
+        assert mismatches(d.copyToHost(ctx), g[key]) == 0

@@ -1,0 +1,136 @@
+"""The int8 path on the GPU: int8 x int8 -> int32 GEMM, per-channel requantisation, and the fused int8 convolution, against the CPU
+oracle of src/layers/Conv2D.cpp:240-308 — BIT FOR BIT (int32 accumulators, requantised int8 outputs and the fp32 outputs of the
+un-fused float tail)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from minml_amd import backend as B
+from minml_amd import core as ml
+from minml_amd.conv2d import Conv2D
+from util import init_for_test, mismatches
+
+pytestmark = pytest.mark.gpu
+
+# the transforms of test/backend/test_quantization.cpp:189-191
+IN_QD, OUT_QD, EXT_QD = (0.123, 4.56), (0.078, 0.9), (0.078, -0.9)
+
+
+def init_for_test_int8(shape, shift):
+    """src/utils/testing_util.cpp:36-40: int8(255 * sin(i / 10 + shift) - 128), wrapped like the C conversion."""
+    n = int(np.prod(shape))
+    i = np.arange(n, dtype=np.float64)
+    v = np.trunc(255.0 * np.sin(i / 10.0 + shift) - 128.0).astype(np.int64)
+    return ((v + 128) % 256 - 128).astype(np.int8).reshape(shape)
+
+
+@pytest.mark.parametrize("shape", [(75, 44, 36), (1716, 44, 36), (130, 70, 64), (300, 256, 2304), (33, 5, 20), (64, 64, 16)])
+def test_int8_gemm_exact(ctx, shape):
+    M, N, K = shape
+    rng = np.random.default_rng(M)
+    A = rng.integers(-128, 128, (M, K)).astype(np.int8)
+    Bm = rng.integers(-128, 128, (N, K)).astype(np.int8)
+    dC = ml.Tensor((M, N), "int32")
+    ml.gemm(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.0, 0.0)
+    assert mismatches(dC.copyToHost(ctx), O.int8_gemm_nt(A, Bm)) == 0
+
+
+def test_reference_test_case_conv2D_1x1(ctx):
+    """test/backend/test_quantization.cpp:173-240 with its deterministic inputs: 11 x 12 x 13 x 36 -> 44, int8 GEMM then
+    quantized_scale_shift_act to int8 and to fp32, ReLU, with an int8 residual."""
+    b, h, w, cin, cout = 11, 12, 13, 36, 44
+    x = init_for_test_int8((b, h, w, cin), 1.0)
+    wt = init_for_test_int8((cout, 1, 1, cin), 0.0)
+    bias = init_for_test((cout,), 1.0)
+    scales = init_for_test((cout,), 1.0, 0.001)
+    ext = init_for_test_int8((b, h, w, cout), 0.0)
+    acc = ml.Tensor((b * h * w, cout), "int32")
+    ml.gemm(ctx, "n", "t", acc, ml.toDevice(ctx, x.reshape(-1, cin)), ml.toDevice(ctx, wt.reshape(cout, cin)), 1.0, 0.0)
+    for code in (O.INT8, O.FLOAT32):
+        out = ml.Tensor((b, h, w, cout), code)
+        ml.quantized_scale_shift_act(ctx, out, OUT_QD, acc, ml.toDevice(ctx, scales), ml.toDevice(ctx, bias), "relu", ml.toDevice(ctx, ext), EXT_QD)
+        want = O.int8_conv2d_forward(x, IN_QD, wt, scales, bias, code, OUT_QD, ext, EXT_QD, O.RELU)
+        assert mismatches(out.copyToHost(ctx), want) == 0
+
+
+@pytest.mark.parametrize("shape,cout,k", [((11, 12, 13, 36), 44, 1), ((3, 12, 13, 32), 44, 5), ((2, 15, 15, 64), 64, 3), ((2, 6, 5, 7), 9, 3),
+                                          ((2, 15, 15, 256), 256, 3), ((1, 19, 19, 48), 20, 3), ((2, 9, 9, 16), 130, 1)])
+@pytest.mark.parametrize("act", ["relu", "linear"])
+def test_int8_convolution_bit_exact(ctx, shape, cout, k, act):
+    """Both device routes — the single fused launch and the reference's three calls (im2row with zero-point padding, int8 GEMM,
+    requantisation: src/layers/Conv2D.cpp:214-239) — to int8 and to fp32, with and without residual."""
+    b, h, w, cin = shape
+    rng = np.random.default_rng(cout * k)
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    wt = rng.integers(-127, 128, (cout, k, k, cin)).astype(np.int8)
+    scales = (rng.random(cout) * 0.002 + 0.0005).astype(np.float32)
+    bias = rng.standard_normal(cout).astype(np.float32)
+    ext = rng.integers(-128, 128, (b, h, w, cout)).astype(np.int8)
+    dx, dw, ds, db, de = (ml.toDevice(ctx, a) for a in (x, wt, scales, bias, ext))
+    for use_ext in (True, False):
+        for code in (O.INT8, O.FLOAT32):
+            want = O.int8_conv2d_forward(x, IN_QD, wt, scales, bias, code, OUT_QD, ext if use_ext else None, EXT_QD, ml.act_of(act))
+            dy = ml.Tensor((b, h, w, cout), code)
+            ml.quantizedConvForward(ctx, dx, IN_QD, dw, ds, db, dy, OUT_QD, de if use_ext else None, EXT_QD, act)
+            assert mismatches(dy.copyToHost(ctx), want) == 0
+        layer = Conv2D(ctx, shape, cout, k, act, True, "int8")
+        layer.setupQuantization(wt, scales, bias, [IN_QD, EXT_QD], OUT_QD, int8_mode="reference")
+        ws = ml.Tensor((max(1, layer.getWorkspaceSize()),), B.DTYPE_INT32)
+        dy = ml.Tensor((b, h, w, cout), "int8")
+        layer.forward([dx, de] if use_ext else [dx], dy, ws)
+        want = O.int8_conv2d_forward(x, IN_QD, wt, scales, bias, O.INT8, OUT_QD, ext if use_ext else None, EXT_QD, ml.act_of(act))
+        assert mismatches(dy.copyToHost(ctx), want) == 0
+
+
+def test_quantized_network_layer_config3(ctx):
+    """Config 3's recipe on one residual-block convolution: per-output-channel symmetric int8 weights (scale = max|w| / 127), per-tensor
+    symmetric activations (shift 0), int32 accumulation, requantisation with fused bias + ReLU. Quantised parameters come from the
+    reference's quantize_weights arithmetic (src/layers/quantization.cpp:55-93)."""
+    rng = np.random.default_rng(33)
+    cin = cout = 256
+    w = (rng.standard_normal((cout, 3, 3, cin)) * np.sqrt(2.0 / (9 * cin))).astype(np.float32)
+    bias = (rng.standard_normal(cout) * 0.01).astype(np.float32)
+    xf = np.maximum(rng.standard_normal((4, 15, 15, cin)), 0).astype(np.float32)
+    in_qd = (float(np.abs(xf).max() / 127.0), 0.0)
+    out_qd = (0.05, 0.0)
+    q, scales, qb = O.quantize_weights(w, bias, in_qd)
+    assert np.array_equal(qb, bias)  # symmetric activations: nothing folded into the bias
+    xq = np.clip(np.round(xf / in_qd[0]), -128, 127).astype(np.int8)
+    dy = ml.Tensor((4, 15, 15, cout), "int8")
+    ml.quantizedConvForward(ctx, ml.toDevice(ctx, xq), in_qd, ml.toDevice(ctx, q), ml.toDevice(ctx, scales), ml.toDevice(ctx, qb), dy, out_qd, None,
+                            (1.0, 0.0), "relu")
+    want = O.int8_conv2d_forward(xq, in_qd, q, scales, qb, O.INT8, out_qd, None, (1.0, 0.0), O.RELU)
+    assert mismatches(dy.copyToHost(ctx), want) == 0
+    # and the quantised layer tracks the fp32 layer it came from
+    ref = O.conv2d_forward(xf, w, bias, None, O.RELU)
+    deq = dy.copyToHost(ctx).astype(np.float32) * out_qd[0]
+    assert np.abs(deq - ref).mean() < 0.05
+
+
+def test_int8_full_size_properties(ctx):
+    """Config 3 at full size (B = 1024, 15x15, 256 -> 256, 3x3): positions are independent (a sub-batch reproduces its slice bit for
+    bit), a sample of positions matches the oracle, and the sum of all int32 accumulators equals the closed form
+    sum_o sum_taps (sum_c w[o,tap,c] * colsum[tap,c]) computed in int64 from column sums of the input."""
+    rng = np.random.default_rng(34)
+    shape, cout = (1024, 15, 15, 256), 256
+    x = rng.integers(-128, 128, shape).astype(np.int8)
+    wt = rng.integers(-127, 128, (cout, 3, 3, 256)).astype(np.int8)
+    scales = np.full(cout, 1.0, np.float32)
+    bias = np.zeros(cout, np.float32)
+    qd = (1.0, 0.0)
+    dx, dw, ds, db = (ml.toDevice(ctx, a) for a in (x, wt, scales, bias))
+    full = ml.Tensor(shape[:3] + (cout,), "float32")
+    ml.quantizedConvForward(ctx, dx, qd, dw, ds, db, full, qd, None, qd, "linear")
+    got = full.copyToHost(ctx)  # float(acc) exactly, |acc| < 2^24 is not guaranteed, so compare through the oracle and sub-batches
+    part = ml.Tensor((8, 15, 15, cout), "float32")
+    ml.quantizedConvForward(ctx, dx.view((8, 15, 15, 256), 500 * 225 * 256), qd, dw, ds, db, part, qd, None, qd, "linear")
+    assert np.array_equal(part.copyToHost(ctx), got[500:508])
+    want = O.int8_conv2d_forward(x[500:502], qd, wt, scales, bias, O.FLOAT32, qd)
+    assert np.array_equal(got[500:502], want)
+    # checksum of the integer accumulators through the int8 GEMM on the 1x1 view (exact int32), against the closed form
+    acc = ml.Tensor((1024 * 225, cout), "int32")
+    w1 = np.ascontiguousarray(wt[:, 1, 1, :])
+    ml.gemm(ctx, "n", "t", acc, dx.view((1024 * 225, 256)), ml.toDevice(ctx, w1), 1.0, 0.0)
+    total = int(acc.copyToHost(ctx).astype(np.int64).sum())
+    colsum = x.reshape(-1, 256).astype(np.int64).sum(axis=0)
+    assert total == int((w1.astype(np.int64) @ colsum).sum())

@@ -1,0 +1,162 @@
+"""Whole-network parity and runtime behaviour on the GPU.
+
+The network is the synthetic residual net of the benchmark configurations run layer by layer through the C-ABI (minml_amd.resnet),
+checked against the CPU execution of the same call sequence (oracle/cpu_net.py) "per layer and at the network head": fp32 within 1e-4,
+fp16 within 1e-2 max-abs relative error."""
+import time
+
+import numpy as np
+import pytest
+
+import oracle as O
+from oracle.cpu_net import CpuResNet
+from minml_amd import backend as B
+from minml_amd import core as ml
+from minml_amd.resnet import ResNet, make_input, make_parameters
+from util import TOL, max_abs_rel, mismatches
+
+pytestmark = pytest.mark.gpu
+
+
+def run_both(ctx, batch, channels, blocks, dtype, seed, chunk=None):
+    conv = O.to_half if dtype == "float16" else (lambda a: np.ascontiguousarray(a, np.float32))
+    params = make_parameters(seed, 32, channels, blocks)
+    x = make_input(seed, batch, 15, 32)
+    net = ResNet(ctx, batch, 15, 32, channels, blocks, dtype, params, conv, chunk=chunk)
+    net.setInput(conv(x))
+    head = net.forward().copyToHost(ctx)
+    trunk = net.trunk_output().copyToHost(ctx)
+    cpu = CpuResNet([(conv(w), conv(b)) for (w, b) in params], blocks, "oracle")
+    want_head, want_trunk = cpu.forward(conv(x), return_trunk=True)
+    return head, trunk, want_head, want_trunk
+
+
+def test_config1_topology_fp32(ctx):
+    """Config 1's topology (stem 32 -> 128, 10 residual blocks x 128, 1x1 policy head, fp32, seed 0) at a batch the oracle finishes."""
+    O.set_num_threads(8)
+    head, trunk, want_head, want_trunk = run_both(ctx, 4, 128, 10, "float32", 0)
+    assert max_abs_rel(trunk, want_trunk) <= 1e-4
+    assert max_abs_rel(head, want_head) <= 1e-4
+
+
+def test_config2_topology_fp16(ctx):
+    """Config 2's topology (20 blocks x 256 channels, fp16 storage, fp32 accumulation, seed 1) at batch 2."""
+    O.set_num_threads(8)
+    head, trunk, want_head, want_trunk = run_both(ctx, 2, 256, 20, "float16", 1)
+    assert max_abs_rel(trunk, want_trunk) <= 1e-2
+    assert max_abs_rel(head, want_head) <= 1e-2
+
+
+def test_per_layer_fp16(ctx):
+    """Every layer of a 3-block fp16 network against the oracle run on the GPU's own input of that layer (no error accumulation)."""
+    rng = np.random.default_rng(2)
+    params = make_parameters(2, 32, 64, 3)
+    x = O.to_half(make_input(2, 3, 15, 32))
+    from minml_amd.conv2d import Conv2D
+
+    cur = x
+    residual = None
+    for idx, (w, b) in enumerate(params[:-1]):
+        wq, bq = O.to_half(w), O.to_half(b)
+        layer = Conv2D(ctx, cur.shape, w.shape[0], 3, "relu", True, "float16")
+        layer.setWeights(wq, bq)
+        ws = ml.Tensor((layer.getWorkspaceSize(),), "float16")
+        out = ml.Tensor(cur.shape[:3] + (w.shape[0],), "float16")
+        use_res = idx > 0 and idx % 2 == 0
+        inputs = [ml.toDevice(ctx, cur)] + ([ml.toDevice(ctx, residual)] if use_res else [])
+        layer.forward(inputs, out, ws)
+        got = out.copyToHost(ctx)
+        v = O.winograd_input_transform(cur)
+        m = O.gemm(v, O.winograd_weight_transform(wq))
+        want = O.winograd_output_transform(m, out.shape, bq, residual if use_res else None, O.RELU)
+        assert max_abs_rel(got, want) <= 1e-2
+        if idx % 2 == 0:
+            residual = got
+        cur = got
+
+
+def test_chunked_execution_is_bit_identical(ctx):
+    """Splitting the batch into cache-resident sub-batches must not change a single bit (positions are independent)."""
+    params = make_parameters(5, 32, 64, 2)
+    x = O.to_half(make_input(5, 12, 15, 32))
+    outs = []
+    for chunk in (12, 4, 5):
+        net = ResNet(ctx, 12, 15, 32, 64, 2, "float16", params, O.to_half, chunk=chunk)
+        net.setInput(x)
+        outs.append(net.forward().copyToHost(ctx))
+    assert mismatches(outs[0], outs[1]) == 0
+    assert mismatches(outs[0], outs[2]) == 0
+
+
+def test_full_size_batch_1024_properties(ctx):
+    """The benchmark workload itself (config 2: B = 1024): repeated passes are bit-identical (no races, no stale workspace), and the
+    first positions reproduce a batch-4 run of the same network bit for bit, which in turn is checked against the oracle."""
+    params = make_parameters(1, 32, 256, 20)
+    x = O.to_half(make_input(1, 1024, 15, 32))
+    net = ResNet(ctx, 1024, 15, 32, 256, 20, "float16", params, O.to_half)
+    net.setInput(x)
+    a = net.forward().copyToHost(ctx)
+    b = net.forward().copyToHost(ctx)
+    assert mismatches(a, b) == 0
+    small = ResNet(ctx, 4, 15, 32, 256, 20, "float16", params, O.to_half)
+    small.setInput(x[:4])
+    c = small.forward().copyToHost(ctx)
+    assert mismatches(a[:4], c) == 0
+    assert np.isfinite(O.from_half(a)).all()
+    O.set_num_threads(8)
+    cpu = CpuResNet([(O.to_half(w), O.to_half(bb)) for (w, bb) in params], 20, "oracle")
+    assert max_abs_rel(c[:1], cpu.forward(x[:1])) <= 1e-2
+
+
+# ---- runtime: context, events, memory ---------------------------------------------------------------------------------------------
+def test_device_identity():
+    assert ml.number_of_devices() >= 1
+    info = B.fn("get_device_info")(0).decode()
+    assert "gfx950" in info
+    assert B.fn("get_memory")(0) > 100000  # MB
+    for dtype, ok in ((B.DTYPE_FLOAT16, True), (B.DTYPE_FLOAT32, True), (B.DTYPE_INT8, True), (B.DTYPE_INT32, True), (B.DTYPE_FLOAT64, False)):
+        assert bool(B.fn("supports_type")(0, dtype)) == ok
+    assert B.fn("get_device_features")(0)
+
+
+def test_memory_calls(ctx):
+    t = ml.Tensor((1000,), "float32")
+    t.setall(ctx, 1.5)
+    assert np.array_equal(t.copyToHost(ctx), np.full(1000, 1.5, np.float32))
+    t.zeroall(ctx)
+    assert not t.copyToHost(ctx).any()
+    h = ml.Tensor((7,), "float16")
+    h.setall(None, 2.0)  # context-less calls are synchronous
+    assert np.array_equal(h.copyToHost(), np.full(7, 0x4000, np.uint16))
+    src = ml.toDevice(ctx, np.arange(100, dtype=np.int32))
+    dst = ml.Tensor((100,), "int32")
+    dst.zeroall(ctx)
+    B.fn("memcpy_within_device")(ctx.handle, dst.ptr, 40, src.ptr, 80, 120)  # 30 ints from src[20:] to dst[10:]
+    got = dst.copyToHost(ctx)
+    assert np.array_equal(got[10:40], np.arange(20, 50)) and not got[:10].any() and not got[40:].any()
+    view = src.view((10,), 90)
+    assert np.array_equal(view.copyToHost(ctx), np.arange(90, 100))
+    with pytest.raises(ValueError):
+        src.view((20,), 90)
+
+
+def test_events_and_context(ctx):
+    x = ml.Tensor((1 << 24,), "float32")
+    start = ml.Event(ctx)
+    for _ in range(10):
+        x.setall(ctx, 1.0)
+    end = ml.Event(ctx)
+    end.synchronize()
+    assert start.isReady() and end.isReady()
+    dt = ml.Event.getElapsedTime(start, end)
+    assert 0.0 < dt < 1.0
+    ctx.synchronize()
+    assert ctx.isReady()
+    other = ml.Context(0)  # a second context = a second stream on the same device
+    y = ml.Tensor((16,), "int32")
+    y.setall(other, 3)
+    other.synchronize()
+    assert np.array_equal(y.copyToHost(other), np.full(16, 3, np.int32))
+    other.destroy()
+    start.destroy()
+    end.destroy()

@@ -1,0 +1,159 @@
+"""Winograd F(4x4,3x3) transforms on the GPU against the CPU oracle, through the C-ABI (hip_winograd_*_transform).
+
+The bar: the three transforms reproduce the reference's expression trees, so fp32 results and truncated fp16 results are compared
+BIT FOR BIT (ReLU / linear); transcendental activations within the per-layer tolerance (max-abs relative 1e-4 fp32, 1e-2 fp16).
+Shapes follow test/backend/test_winograd.cpp:396-513 ({3,9,11,35}, {3,7,11,35}: edge tiles, channel counts that match no vector width)
+plus the benchmark's own (15x15 x 256, 19x19)."""
+import numpy as np
+import pytest
+
+import oracle as O
+from minml_amd import core as ml
+from util import TOL, max_abs_rel, mismatches, random_tensor
+from test_oracle_pins import INPUT_ONES, INPUT_RAMP, OUTPUT_ONES, OUTPUT_RAMP, WEIGHT_NINES, WEIGHT_RAMP, both_channels
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [((3, 9, 11, 35), 21), ((3, 7, 11, 35), 35), ((2, 15, 15, 32), 64), ((2, 15, 15, 256), 256), ((1, 19, 19, 64), 128), ((1, 4, 4, 2), 2),
+          ((2, 3, 2, 1), 1), ((1, 5, 17, 6), 10)]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("shape,cout", SHAPES)
+def test_transforms_bit_exact(ctx, dtype, shape, cout):
+    rng = np.random.default_rng(hash((shape, cout)) % 2 ** 31)
+    b, h, w, c = shape
+    tiles = b * ((h + 3) // 4) * ((w + 3) // 4)
+    # weights
+    wt = random_tensor(rng, (cout, 3, 3, c), dtype)
+    dm = ml.Tensor((36, cout, c), dtype)
+    for invert in (False, True):
+        ml.winogradWeightTransform(ctx, ml.toDevice(ctx, wt), dm, invert)
+        assert mismatches(dm.copyToHost(ctx), O.winograd_weight_transform(wt, invert)) == 0
+    # input
+    x = random_tensor(rng, shape, dtype)
+    dv = ml.Tensor((36, tiles, c), dtype)
+    ml.winogradInputTransform(ctx, (cout, 3, 3, c), ml.toDevice(ctx, x), dv)
+    assert mismatches(dv.copyToHost(ctx), O.winograd_input_transform(x)) == 0
+    # output with every combination of bias / residual, linear and ReLU
+    m = random_tensor(rng, (36, tiles, cout), dtype)
+    bias = random_tensor(rng, (cout,), dtype)
+    ext = random_tensor(rng, (b, h, w, cout), dtype)
+    dmm, db, de = ml.toDevice(ctx, m), ml.toDevice(ctx, bias), ml.toDevice(ctx, ext)
+    for use_bias in (True, False):
+        for use_ext in (True, False):
+            for act in (O.LINEAR, O.RELU):
+                dy = ml.Tensor((b, h, w, cout), dtype)
+                dy.setall(ctx, 7.0)
+                ml.winogradOutputTransform(ctx, (cout, 3, 3, cout), dmm, dy, db if use_bias else None, de if use_ext else None, act)
+                want = O.winograd_output_transform(m, (b, h, w, cout), bias if use_bias else None, ext if use_ext else None, act)
+                assert mismatches(dy.copyToHost(ctx), want) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("act", [O.SIGMOID, O.TANH, O.LEAKY_RELU, O.EXP])
+def test_output_transform_other_activations(ctx, dtype, act):
+    rng = np.random.default_rng(act)
+    shape, cout = (2, 9, 11, 12), 12
+    m = random_tensor(rng, (36, 2 * 3 * 3, cout), dtype, 0.2)
+    bias = random_tensor(rng, (cout,), dtype)
+    ext = random_tensor(rng, shape, dtype)
+    dy = ml.Tensor(shape, dtype)
+    ml.winogradOutputTransform(ctx, (cout, 3, 3, cout), ml.toDevice(ctx, m), dy, ml.toDevice(ctx, bias), ml.toDevice(ctx, ext), act)
+    assert max_abs_rel(dy.copyToHost(ctx), O.winograd_output_transform(m, shape, bias, ext, act)) <= TOL[dtype]
+
+
+def test_golden_vectors_through_the_gpu(ctx):
+    """The literals of test/backend/test_winograd.cpp:218-323, mean-abs-diff <= 1e-4 as there."""
+    for image, expected in ((np.ones((4, 4)), INPUT_ONES), (np.arange(1, 17).reshape(4, 4), INPUT_RAMP)):
+        dv = ml.Tensor((36, 1, 2), "float32")
+        ml.winogradInputTransform(ctx, (2, 3, 3, 2), ml.toDevice(ctx, both_channels(image)[None]), dv)
+        got = dv.copyToHost(ctx)
+        for ch in range(2):
+            assert np.abs(got[:, 0, ch].reshape(6, 6) - np.array(expected)).mean() <= 1e-4
+    for matrices, expected in ((np.ones(36), OUTPUT_ONES), (np.arange(1, 37), OUTPUT_RAMP)):
+        dy = ml.Tensor((1, 4, 4, 2), "float32")
+        ml.winogradOutputTransform(ctx, (2, 3, 3, 2), ml.toDevice(ctx, both_channels(matrices)[:, None, :]), dy, None, None, "linear")
+        got = dy.copyToHost(ctx)
+        for ch in range(2):
+            assert np.abs(got[0, :, :, ch] - np.array(expected)).mean() <= 1e-4
+    for kernel, expected in ((np.full((3, 3), 9.0), WEIGHT_NINES), (np.arange(1, 10).reshape(3, 3), WEIGHT_RAMP)):
+        dm = ml.Tensor((36, 1, 2), "float32")
+        ml.winogradWeightTransform(ctx, ml.toDevice(ctx, both_channels(kernel)[None]), dm, False)
+        got = dm.copyToHost(ctx)
+        for ch in range(2):
+            assert np.abs(got[:, 0, ch].reshape(6, 6) - np.array(expected)).mean() <= 1e-4
+
+
+@pytest.mark.parametrize("tag,dtype", [("f32", "float32"), ("f16", "float16")])
+def test_reference_fixtures_through_the_gpu(ctx, golden, tag, dtype):
+    """Outputs recorded from the reference's compiled CPU backend (tests/golden/make_fixtures.py)."""
+    g = golden
+    dm = ml.Tensor((36, 13, 19), dtype)
+    ml.winogradWeightTransform(ctx, ml.toDevice(ctx, g["wg_w_" + tag]), dm, False)
+    assert mismatches(dm.copyToHost(ctx), g["wg_wm_" + tag]) == 0
+    ml.winogradWeightTransform(ctx, ml.toDevice(ctx, g["wg_w_" + tag]), dm, True)
+    assert mismatches(dm.copyToHost(ctx), g["wg_wm_inverted_" + tag]) == 0
+    dv = ml.Tensor((36, 18, 19), dtype)
+    ml.winogradInputTransform(ctx, (13, 3, 3, 19), ml.toDevice(ctx, g["wg_x_" + tag]), dv)
+    assert mismatches(dv.copyToHost(ctx), g["wg_v_" + tag]) == 0
+    dy = ml.Tensor((2, 9, 11, 13), dtype)
+    ml.winogradOutputTransform(ctx, (13, 3, 3, 13), ml.toDevice(ctx, g["wg_m_" + tag]), dy, ml.toDevice(ctx, g["wg_bias_" + tag]),
+                               ml.toDevice(ctx, g["wg_ext_" + tag]), "relu")
+    assert mismatches(dy.copyToHost(ctx), g["wg_y_relu_" + tag]) == 0
+    ml.winogradOutputTransform(ctx, (13, 3, 3, 13), ml.toDevice(ctx, g["wg_m_" + tag]), dy, ml.toDevice(ctx, g["wg_bias_" + tag]), None, "linear")
+    assert mismatches(dy.copyToHost(ctx), g["wg_y_linear_" + tag]) == 0
+    # the GEMM in between, within tolerance (the MFMA accumulation order is the hardware's)
+    dmo = ml.Tensor((36, 18, 13), dtype)
+    ml.gemmBatched(ctx, "n", "t", dmo, ml.toDevice(ctx, g["wg_v_" + tag]), ml.toDevice(ctx, g["wg_wm_" + tag]))
+    assert max_abs_rel(dmo.copyToHost(ctx), g["wg_m_" + tag]) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_full_pipeline_against_direct_convolution(ctx, dtype):
+    """test/backend/test_conv2D.cpp:580-629: {3,13,17,35} -> 21 filters, weight transform -> input transform -> gemmBatched('n','t') ->
+    output transform with bias, against the direct convolution."""
+    rng = np.random.default_rng(11)
+    x = random_tensor(rng, (3, 13, 17, 35), dtype)
+    w = random_tensor(rng, (21, 3, 3, 35), dtype, 0.1)
+    bias = random_tensor(rng, (21,), dtype)
+    wm = ml.Tensor((36, 21, 35), dtype)
+    ml.winogradWeightTransform(ctx, ml.toDevice(ctx, w), wm, False)
+    v = ml.Tensor((36, 3 * 4 * 5, 35), dtype)
+    m = ml.Tensor((36, 3 * 4 * 5, 21), dtype)
+    ml.winogradInputTransform(ctx, (21, 3, 3, 35), ml.toDevice(ctx, x), v)
+    ml.gemmBatched(ctx, "n", "t", m, v, wm, 1.0, 0.0)
+    y = ml.Tensor((3, 13, 17, 21), dtype)
+    ml.winogradOutputTransform(ctx, (21, 3, 3, 35), m, y, ml.toDevice(ctx, bias), None, "sigmoid")
+    got = y.copyToHost(ctx)
+    direct = O.conv2d_forward(x, w, bias, None, O.SIGMOID)
+    if dtype == "float32":
+        assert max_abs_rel(got, direct) <= TOL[dtype]
+    else:
+        # in fp16 the Winograd algorithm itself (matrices truncated to half between the stages) is what differs from a direct
+        # convolution, on the CPU reference as much as here: the tolerance applies against the same algorithm on the CPU, and the
+        # distance to the direct convolution is bounded the way the reference bounds it (mean absolute difference)
+        pipeline = O.winograd_output_transform(O.gemm(O.winograd_input_transform(x), O.winograd_weight_transform(w)), (3, 13, 17, 21), bias, None,
+                                               O.SIGMOID)
+        assert max_abs_rel(got, pipeline) <= TOL[dtype]
+        assert np.abs(O.from_half(got) - O.from_half(direct)).mean() <= 1e-2
+
+
+def test_empty_and_full_size_properties(ctx):
+    """Empty batch is a no-op; at the benchmark's full size (B = 1024, 15x15, 256 channels, fp16) the transform of a batch equals the
+    transforms of its halves (positions are independent), and an all-zero image transforms to zeros."""
+    ml.winogradInputTransform(ctx, (8, 3, 3, 8), ml.Tensor((0, 15, 15, 8), "float16"), ml.Tensor((36, 0, 8), "float16"))
+    rng = np.random.default_rng(12)
+    x = random_tensor(rng, (1024, 15, 15, 256), "float16")
+    dx = ml.toDevice(ctx, x)
+    full = ml.Tensor((36, 16384, 256), "float16")
+    ml.winogradInputTransform(ctx, (256, 3, 3, 256), dx, full)
+    got = full.copyToHost(ctx)
+    half = ml.Tensor((36, 8192, 256), "float16")
+    ml.winogradInputTransform(ctx, (256, 3, 3, 256), dx.view((512, 15, 15, 256), 512 * 225 * 256), half)
+    assert np.array_equal(got[:, 8192:], half.copyToHost(ctx))
+    sample = O.winograd_input_transform(x[1000:1002])
+    assert np.array_equal(got[:, 16000:16032], sample)
+    dx.zeroall(ctx)
+    ml.winogradInputTransform(ctx, (256, 3, 3, 256), dx, full)
+    assert not full.copyToHost(ctx).any()

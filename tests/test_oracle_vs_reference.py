@@ -1,0 +1,111 @@
+"""The CPU oracle against the reference itself: (1) the committed fixtures that the reference's compiled CPU backend produced
+(tests/golden/make_fixtures.py) — runs everywhere; (2) the compiled reference library oracle/_ref where it has been built — bit for bit
+on fresh random inputs, in fp32 and fp16, including the reference's split of K at 1024."""
+import numpy as np
+import pytest
+
+import oracle as O
+from util import mismatches, random_tensor
+
+needs_ref = pytest.mark.skipif(O.reference() is None, reason="oracle/_ref (compiled reference CPU backend) is not built here")
+
+
+@pytest.mark.parametrize("tag", ["f32", "f16"])
+def test_fixtures_winograd(golden, tag):
+    g = golden
+    assert mismatches(O.winograd_weight_transform(g["wg_w_" + tag]), g["wg_wm_" + tag]) == 0
+    assert mismatches(O.winograd_weight_transform(g["wg_w_" + tag], True), g["wg_wm_inverted_" + tag]) == 0
+    assert mismatches(O.winograd_input_transform(g["wg_x_" + tag]), g["wg_v_" + tag]) == 0
+    assert mismatches(O.gemm(g["wg_v_" + tag], g["wg_wm_" + tag]), g["wg_m_" + tag]) == 0
+    y = O.winograd_output_transform(g["wg_m_" + tag], (2, 9, 11, 13), g["wg_bias_" + tag], g["wg_ext_" + tag], O.RELU)
+    assert mismatches(y, g["wg_y_relu_" + tag]) == 0
+    assert mismatches(O.winograd_output_transform(g["wg_m_" + tag], (2, 9, 11, 13), g["wg_bias_" + tag]), g["wg_y_linear_" + tag]) == 0
+
+
+@pytest.mark.parametrize("tag", ["f32", "f16"])
+def test_fixtures_gemm_and_conv(golden, tag):
+    g = golden
+    d = O.gemm(g["ge_a_" + tag], g["ge_b_" + tag], alpha=1.1, beta=0.1, C=g["ge_c_" + tag], bias=g["ge_bias_" + tag], act=O.RELU)
+    assert mismatches(d, g["ge_d_" + tag]) == 0
+    assert mismatches(O.gemm(g["gk_a_" + tag], g["gk_b_" + tag]), g["gk_d_" + tag]) == 0  # K = 1200 > 1024: two K tiles
+    assert mismatches(O.im2row(g["cv_x_" + tag], 5), g["cv_rows_" + tag]) == 0
+    y = O.conv2d_forward(g["cv_x_" + tag], g["cv_w_" + tag], g["cv_bias_" + tag], g["cv_add_" + tag], O.RELU)
+    assert mismatches(y, g["cv_y_" + tag]) == 0
+    got = O.add_bias_act(g["cv_x_" + tag], None, O.LINEAR)
+    assert mismatches(got, g["cv_x_" + tag]) == 0
+
+
+def test_fixtures_unpack_and_convert(golden):
+    g = golden
+    assert mismatches(O.unpack_input(g["up_packed"], (3, 5, 40), O.FLOAT32), g["up_f32"]) == 0
+    assert mismatches(O.unpack_input(g["up_packed"], (3, 5, 40), O.FLOAT16), g["up_f16"]) == 0
+    ours, theirs = O.to_half(g["cvt_src"]), g["cvt_f16"]
+    # the reference's vector narrowing (vcvtps2ph, round toward zero) saturates to the largest finite half where the scalar table method
+    # that the oracle restates (src/backend/cpu/fp16.hpp:61-68) gives infinity; everywhere else the two agree bit for bit
+    finite = np.abs(g["cvt_src"]) < 65504.0
+    assert mismatches(ours[finite], theirs[finite]) == 0
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_reference_bit_exact(dtype):
+    ref = O.reference()
+    rng = np.random.default_rng(0)
+    for shape, cout in (((3, 9, 11, 35), 21), ((3, 7, 11, 35), 35), ((1, 15, 15, 32), 16)):
+        c = shape[3]
+        w = random_tensor(rng, (cout, 3, 3, c), dtype)
+        x = random_tensor(rng, shape, dtype)
+        assert mismatches(O.winograd_weight_transform(w), ref.winograd_weight_transform(w)) == 0
+        assert mismatches(O.winograd_weight_transform(w, True), ref.winograd_weight_transform(w, True)) == 0
+        v = O.winograd_input_transform(x)
+        assert mismatches(v, ref.winograd_input_transform(x)) == 0
+        u = O.winograd_weight_transform(w)
+        m = O.gemm(v, u)
+        assert mismatches(m, ref.gemm_batched(v, u)) == 0
+        out_shape = shape[:3] + (cout,)
+        bias = random_tensor(rng, (cout,), dtype)
+        ext = random_tensor(rng, out_shape, dtype)
+        for act in (O.LINEAR, O.RELU, O.SIGMOID, O.TANH):
+            assert mismatches(O.winograd_output_transform(m, out_shape, bias, ext, act), ref.winograd_output_transform(m, out_shape, bias, ext, act)) == 0
+        if cout % 16 == 0:  # bias-less calls are only well defined in the reference for channel counts that skip its scalar tail loop
+            assert mismatches(O.winograd_output_transform(m, out_shape), ref.winograd_output_transform(m, out_shape)) == 0
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_reference_gemm_and_conv_bit_exact(dtype):
+    ref = O.reference()
+    rng = np.random.default_rng(1)
+    for ops in ("nn", "nt", "tn", "tt"):
+        A = random_tensor(rng, (30, 40) if ops[0] == "n" else (40, 30), dtype)
+        Bm = random_tensor(rng, (40, 20) if ops[1] == "n" else (20, 40), dtype)
+        assert mismatches(O.gemm(A, Bm, ops[0], ops[1], alpha=1.1), ref.gemm_ex(A, Bm, ops[0], ops[1], alpha=1.1)) == 0
+    A = random_tensor(rng, (50, 2304), dtype, 0.1)
+    Bm = random_tensor(rng, (20, 2304), dtype, 0.1)
+    bias = random_tensor(rng, (20,), dtype)
+    C = random_tensor(rng, (50, 20), dtype)
+    got = O.gemm(A, Bm, alpha=0.7, beta=1.0, C=C, bias=bias, act=O.RELU)
+    assert mismatches(got, ref.gemm_ex(A, Bm, alpha=0.7, beta=1.0, C=C, bias=bias, act=O.RELU)) == 0
+    x = random_tensor(rng, (2, 7, 6, 128), dtype)
+    w = random_tensor(rng, (24, 5, 5, 128), dtype, 0.1)
+    b = random_tensor(rng, (24,), dtype)
+    add = random_tensor(rng, (2, 7, 6, 24), dtype)
+    assert mismatches(O.conv2d_forward(x, w, b, add, O.SIGMOID), ref.conv2d_forward(x, w, b, add, O.SIGMOID)) == 0
+    assert mismatches(O.im2row(x, 5), ref.im2row(x, 5)) == 0
+    bb = random_tensor(rng, (128,), dtype)
+    assert mismatches(O.add_bias_act(x, bb, O.RELU), ref.add_bias_act(x, bb, O.RELU)) == 0
+
+
+@needs_ref
+def test_reference_network_bit_exact():
+    """A 2-block network end to end: the oracle engine and the reference engine of oracle/cpu_net.py agree bit for bit."""
+    from oracle.cpu_net import CpuResNet
+    from minml_amd.resnet import make_input, make_parameters
+
+    params = make_parameters(3, 32, 48, 2)
+    x = make_input(3, 3, 15, 32)
+    for conv in (lambda a: a, O.to_half):
+        ps = [(conv(w), conv(b)) for (w, b) in params]
+        a = CpuResNet(ps, 2, "oracle").forward(conv(x))
+        b = CpuResNet(ps, 2, "reference").forward(conv(x))
+        assert mismatches(a, b) == 0
