@@ -136,48 +136,89 @@ namespace
 		}
 	}
 
-	/* input [B][H][W][C] -> matrices [36][B*tiles_h*tiles_w][C] */
+	/* VEC storage elements moved by one load instruction and kept unconverted until they are needed */
+	template<typename T, int N>
+	struct RawVec
+	{
+			typedef T type __attribute__((ext_vector_type(N)));
+			__device__ static __forceinline__ float get(const type &r, int i)
+			{
+				return static_cast<float>(r[i]);
+			}
+	};
+	template<typename T>
+	struct RawVec<T, 1>
+	{
+			typedef T type;
+			__device__ static __forceinline__ float get(const type &r, int)
+			{
+				return static_cast<float>(r);
+			}
+	};
+
+	/*
+	 * input [B][H][W][C] -> matrices [36][B*tiles_h*tiles_w][C]
+	 * All 36 loads of a tile are issued back to back, unconditionally, from coordinates clamped into the image; elements that lie outside
+	 * are replaced by zero afterwards. (A load under a bounds test would sit in its own basic block and be waited for on its own, which
+	 * leaves one 512-byte request in flight per wavefront.) Offsets are 32-bit element offsets from the tensor base.
+	 */
 	template<typename T, int VEC>
 	__global__ __launch_bounds__(256) void kernel_input_transform_4x4_3x3(const T *__restrict__ input, T *__restrict__ matrices, int batch_size,
 			int height, int width, int channels, int tiles_h, int tiles_w)
 	{
-		const int groups = channels / VEC;
-		const int tiles_per_image = tiles_h * tiles_w;
-		const size_t nb_of_tiles = static_cast<size_t>(batch_size) * tiles_per_image;
-		const size_t total = nb_of_tiles * groups;
+		typedef typename RawVec<T, VEC>::type raw_t;
+		const unsigned int groups = channels / VEC;
+		const unsigned int tiles_per_image = tiles_h * tiles_w;
+		const unsigned int nb_of_tiles = batch_size * tiles_per_image;
+		const unsigned int total = nb_of_tiles * groups;
 
 		const unsigned int block = xcd_contiguous_block_id(blockIdx.x, gridDim.x);
-		const size_t gid = static_cast<size_t>(block) * blockDim.x + threadIdx.x;
+		const unsigned int gid = block * blockDim.x + threadIdx.x;
 		if (gid >= total)
 			return;
-		const size_t tile_idx = gid / groups;
-		const int channel = static_cast<int>(gid % groups) * VEC;
+		const unsigned int tile_idx = gid / groups;
+		const unsigned int channel = (gid - tile_idx * groups) * VEC;
 
-		const int batch = static_cast<int>(tile_idx / tiles_per_image);
-		const int in_image = static_cast<int>(tile_idx % tiles_per_image);
-		const int x0 = 4 * (in_image / tiles_w) - 1;
-		const int y0 = 4 * (in_image % tiles_w) - 1;
+		const unsigned int batch = tile_idx / tiles_per_image;
+		const unsigned int in_image = tile_idx - batch * tiles_per_image;
+		const int tile_x = in_image / tiles_w;
+		const int x0 = 4 * tile_x - 1;
+		const int y0 = 4 * (in_image - tile_x * tiles_w) - 1;
 
-		const T *src = input + static_cast<size_t>(batch) * height * width * channels + channel;
+		unsigned int row_offset[6], col_offset[6];
+		bool row_valid[6], col_valid[6];
+#pragma unroll
+		for (int i = 0; i < 6; i++)
+		{
+			const int x = x0 + i;
+			const int y = y0 + i;
+			row_valid[i] = (x >= 0) && (x < height);
+			col_valid[i] = (y >= 0) && (y < width);
+			const int xc = min(max(x, 0), height - 1);
+			const int yc = min(max(y, 0), width - 1);
+			row_offset[i] = (batch * height + xc) * width * channels;
+			col_offset[i] = yc * channels + channel;
+		}
+
+		raw_t raw[6][6];
+#pragma unroll
+		for (int row = 0; row < 6; row++)
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+				raw[row][col] = *reinterpret_cast<const raw_t*>(input + (row_offset[row] + col_offset[col]));
 
 		float tmp[6][6][VEC]; /* [row after the column pass][col] */
 #pragma unroll
 		for (int col = 0; col < 6; col++)
 		{
-			const int y = y0 + col;
 			float line[6][VEC];
 #pragma unroll
 			for (int row = 0; row < 6; row++)
 			{
-				const int x = x0 + row;
-				Vec<T, VEC> tmpv;
-				if (x >= 0 && x < height && y >= 0 && y < width)
-					tmpv.load(src + (static_cast<size_t>(x) * width + y) * channels);
-				else
-					tmpv.zero();
+				const bool valid = row_valid[row] && col_valid[col];
 #pragma unroll
 				for (int c = 0; c < VEC; c++)
-					line[row][c] = tmpv.v[c];
+					line[row][c] = valid ? RawVec<T, VEC>::get(raw[row][col], c) : 0.0f;
 			}
 			float res[6][VEC];
 			input_transform_1d<VEC>(line, res);
@@ -188,8 +229,8 @@ namespace
 					tmp[row][col][c] = res[row][c];
 		}
 
-		T *dst = matrices + tile_idx * channels + channel;
-		const size_t matrix_stride = nb_of_tiles * channels;
+		T *dst = matrices + static_cast<size_t>(tile_idx) * channels + channel;
+		const size_t matrix_stride = static_cast<size_t>(nb_of_tiles) * channels;
 #pragma unroll
 		for (int row = 0; row < 6; row++)
 		{
@@ -207,30 +248,67 @@ namespace
 		}
 	}
 
-	/* matrices [36][B*tiles_h*tiles_w][C] (+ bias [C], + ext [B][H][W][C]) -> output [B][H][W][C] */
-	template<typename T, int VEC>
+	/*
+	 * matrices [36][B*tiles_h*tiles_w][C] (+ bias [C], + ext [B][H][W][C]) -> output [B][H][W][C]
+	 * ACT: 0 = linear, 1 = ReLU (both fused as the reference fuses them), 2 = any other activation, selected at run time.
+	 * The 36 matrix rows and the 16 residual vectors (from clamped coordinates) are requested before any arithmetic.
+	 */
+	template<typename T, int VEC, int ACT, bool HAS_EXT>
 	__global__ __launch_bounds__(256) void kernel_output_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
 			const T *ext, int act, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
 	{
-		const int groups = channels / VEC;
-		const int tiles_per_image = tiles_h * tiles_w;
-		const size_t nb_of_tiles = static_cast<size_t>(batch_size) * tiles_per_image;
-		const size_t total = nb_of_tiles * groups;
+		typedef typename RawVec<T, VEC>::type raw_t;
+		const unsigned int groups = channels / VEC;
+		const unsigned int tiles_per_image = tiles_h * tiles_w;
+		const unsigned int nb_of_tiles = batch_size * tiles_per_image;
+		const unsigned int total = nb_of_tiles * groups;
 
 		const unsigned int block = xcd_contiguous_block_id(blockIdx.x, gridDim.x);
-		const size_t gid = static_cast<size_t>(block) * blockDim.x + threadIdx.x;
+		const unsigned int gid = block * blockDim.x + threadIdx.x;
 		if (gid >= total)
 			return;
-		const size_t tile_idx = gid / groups;
-		const int channel = static_cast<int>(gid % groups) * VEC;
+		const unsigned int tile_idx = gid / groups;
+		const unsigned int channel = (gid - tile_idx * groups) * VEC;
 
-		const int batch = static_cast<int>(tile_idx / tiles_per_image);
-		const int in_image = static_cast<int>(tile_idx % tiles_per_image);
-		const int x0 = 4 * (in_image / tiles_w);
-		const int y0 = 4 * (in_image % tiles_w);
+		const unsigned int batch = tile_idx / tiles_per_image;
+		const unsigned int in_image = tile_idx - batch * tiles_per_image;
+		const int tile_x = in_image / tiles_w;
+		const int x0 = 4 * tile_x;
+		const int y0 = 4 * (in_image - tile_x * tiles_w);
 
-		const T *src = matrices + tile_idx * channels + channel;
-		const size_t matrix_stride = nb_of_tiles * channels;
+		const T *src = matrices + static_cast<size_t>(tile_idx) * channels + channel;
+		const size_t matrix_stride = static_cast<size_t>(nb_of_tiles) * channels;
+		raw_t raw[6][6];
+#pragma unroll
+		for (int row = 0; row < 6; row++)
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+				raw[row][col] = *reinterpret_cast<const raw_t*>(src + static_cast<size_t>(row * 6 + col) * matrix_stride);
+
+		unsigned int offset[4][4]; /* element offsets of the 4x4 outputs, clamped into the image */
+#pragma unroll
+		for (int row = 0; row < 4; row++)
+#pragma unroll
+			for (int col = 0; col < 4; col++)
+			{
+				const int xc = min(x0 + row, height - 1);
+				const int yc = min(y0 + col, width - 1);
+				offset[row][col] = ((batch * height + xc) * width + yc) * channels + channel;
+			}
+		raw_t residual[4][4];
+		if constexpr (HAS_EXT)
+		{
+#pragma unroll
+			for (int row = 0; row < 4; row++)
+#pragma unroll
+				for (int col = 0; col < 4; col++)
+					residual[row][col] = *reinterpret_cast<const raw_t*>(ext + offset[row][col]);
+		}
+		Vec<T, VEC> b;
+		if (bias != nullptr)
+			b.load(bias + channel);
+		else
+			b.zero();
 
 		float tmp[4][6][VEC];
 #pragma unroll
@@ -239,13 +317,9 @@ namespace
 			float line[6][VEC];
 #pragma unroll
 			for (int row = 0; row < 6; row++)
-			{
-				Vec<T, VEC> tmpv;
-				tmpv.load(src + static_cast<size_t>(row * 6 + col) * matrix_stride);
 #pragma unroll
 				for (int c = 0; c < VEC; c++)
-					line[row][c] = tmpv.v[c];
-			}
+					line[row][c] = RawVec<T, VEC>::get(raw[row][col], c);
 			float res[4][VEC];
 			output_transform_1d<VEC>(line, res);
 #pragma unroll
@@ -255,57 +329,33 @@ namespace
 					tmp[row][col][c] = res[row][c];
 		}
 
-		Vec<T, VEC> b;
-		if (bias != nullptr)
-			b.load(bias + channel);
-		else
-			b.zero();
-
-		const size_t image_offset = static_cast<size_t>(batch) * height * width * channels + channel;
 #pragma unroll
 		for (int row = 0; row < 4; row++)
 		{
 			float res[4][VEC];
 			output_transform_1d<VEC>(tmp[row], res);
-			const int x = x0 + row;
 #pragma unroll
 			for (int col = 0; col < 4; col++)
 			{
-				const int y = y0 + col;
-				if (x < height && y < width)
+				Vec<T, VEC> out;
+#pragma unroll
+				for (int c = 0; c < VEC; c++)
 				{
-					const size_t offset = image_offset + (static_cast<size_t>(x) * width + y) * channels;
-					Vec<T, VEC> out;
-#pragma unroll
-					for (int c = 0; c < VEC; c++)
-						out.v[c] = res[col][c] + b.v[c];
-					if (ext != nullptr)
-					{
-						Vec<T, VEC> e;
-						e.load(ext + offset);
-#pragma unroll
-						for (int c = 0; c < VEC; c++)
-							out.v[c] = out.v[c] + e.v[c];
-					}
-					if (act == ACTIVATION_RELU)
-					{
-#pragma unroll
-						for (int c = 0; c < VEC; c++)
-							out.v[c] = fmaxf(out.v[c], 0.0f);
-					}
-					else if (act != ACTIVATION_LINEAR)
+					float t = res[col][c] + b.v[c];
+					if constexpr (HAS_EXT)
+						t = t + RawVec<T, VEC>::get(residual[row][col], c);
+					if constexpr (ACT == 1)
+						t = fmaxf(t, 0.0f);
+					if constexpr (ACT == 2)
 					{ /* the reference stores y and then runs the activation over it: round through the storage type in between */
-#pragma unroll
-						for (int c = 0; c < VEC; c++)
-						{
-							float t = out.v[c];
-							if constexpr (sizeof(T) == 2)
-								t = half_bits_to_float(half_bits_rtz(t));
-							out.v[c] = activate(act, t);
-						}
+						if constexpr (sizeof(T) == 2)
+							t = half_bits_to_float(half_bits_rtz(t));
+						t = activate(act, t);
 					}
-					out.store(output + offset);
+					out.v[c] = t;
 				}
+				if ((x0 + row) < height && (y0 + col) < width)
+					out.store(output + offset[row][col]);
 			}
 		}
 	}
@@ -378,6 +428,34 @@ namespace
 		}
 		MLHIP_CHECK(hipGetLastError());
 	}
+	template<typename T, int VEC>
+	void launch_output_vec(hipStream_t stream, dim3 grid, const T *in, T *out, const T *b, const T *e, int act, int batch, int height, int width,
+			int channels, int tiles_h, int tiles_w)
+	{
+		const dim3 block(256);
+		const int mode = (act == ACTIVATION_LINEAR) ? 0 : ((act == ACTIVATION_RELU) ? 1 : 2);
+#define MLHIP_LAUNCH_OUTPUT(MODE, EXT) \
+		hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, VEC, MODE, EXT>), grid, block, 0, stream, in, out, b, e, act, batch, height, width, channels, tiles_h, tiles_w)
+		if (e != nullptr)
+		{
+			if (mode == 0)
+				MLHIP_LAUNCH_OUTPUT(0, true);
+			else if (mode == 1)
+				MLHIP_LAUNCH_OUTPUT(1, true);
+			else
+				MLHIP_LAUNCH_OUTPUT(2, true);
+		}
+		else
+		{
+			if (mode == 0)
+				MLHIP_LAUNCH_OUTPUT(0, false);
+			else if (mode == 1)
+				MLHIP_LAUNCH_OUTPUT(1, false);
+			else
+				MLHIP_LAUNCH_OUTPUT(2, false);
+		}
+#undef MLHIP_LAUNCH_OUTPUT
+	}
 	template<typename T>
 	void launch_output(hipStream_t stream, const mlTensor_t &matrices, const mlTensor_t &bias, const mlTensor_t &ext, mlTensor_t &y, mlActivationType_t act)
 	{
@@ -385,7 +463,6 @@ namespace
 		const int tiles_h = ceil_div(height, 4), tiles_w = ceil_div(width, 4);
 		const size_t tiles = static_cast<size_t>(batch) * tiles_h * tiles_w;
 		const int vec = pick_vec(channels, matrices.data, y.data, bias.data, ext.data, sizeof(T));
-		const dim3 block(256);
 		const dim3 grid(grid_for(tiles * (channels / vec)));
 		const T *in = ptr<const T>(matrices);
 		T *out = ptr<T>(y);
@@ -395,13 +472,13 @@ namespace
 		switch (vec)
 		{
 			case 4:
-				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 4>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				launch_output_vec<T, 4>(stream, grid, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
 				break;
 			case 2:
-				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 2>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				launch_output_vec<T, 2>(stream, grid, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
 				break;
 			default:
-				hipLaunchKernelGGL((kernel_output_transform_4x4_3x3<T, 1>), grid, block, 0, stream, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
+				launch_output_vec<T, 1>(stream, grid, in, out, b, e, a, batch, height, width, channels, tiles_h, tiles_w);
 				break;
 		}
 		MLHIP_CHECK(hipGetLastError());
@@ -444,6 +521,7 @@ extern "C"
 				"Winograd input transform: matrices must be [36, B*ceil(H/4)*ceil(W/4), C]");
 		if (tiles == 0 || x.dim[3] == 0)
 			return;
+		MLHIP_REQUIRE(volume(x) <= 0xffffffffu && tiles * x.dim[3] <= 0xffffffffu, "Winograd input transform: tensor too large for 32-bit element offsets");
 		MLHIP_REQUIRE(x.data != nullptr && matrices.data != nullptr, "Winograd input transform: null tensor");
 		mlTensor_t m = matrices;
 		if (x.dtype == DTYPE_FLOAT16)
@@ -466,6 +544,7 @@ extern "C"
 			MLHIP_REQUIRE(ext.dtype == y.dtype && volume(ext) == volume(y), "Winograd output transform: ext must have the output's shape and dtype");
 		if (tiles == 0 || y.dim[3] == 0)
 			return;
+		MLHIP_REQUIRE(volume(y) <= 0xffffffffu && tiles * y.dim[3] <= 0xffffffffu, "Winograd output transform: tensor too large for 32-bit element offsets");
 		MLHIP_REQUIRE(y.data != nullptr && matrices.data != nullptr, "Winograd output transform: null tensor");
 		mlTensor_t out = y;
 		if (y.dtype == DTYPE_FLOAT16)
