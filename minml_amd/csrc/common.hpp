@@ -60,6 +60,8 @@ namespace mlhip
 	}
 	/* returns device scratch of at least `bytes` bytes; grows by reallocating after the stream has drained */
 	void* get_workspace(mlContext_t context, size_t bytes);
+	/* number of compute units of the current device (cached per device) */
+	int device_compute_units();
 
 	inline int size_of(mlDataType_t dtype)
 	{

@@ -16,6 +16,7 @@
 #include "gemm_core.hpp"
 #include "epilogues.hpp"
 #include "gemm_launch.hpp"
+#include "gemm_stream.hpp"
 
 namespace
 {
@@ -79,6 +80,35 @@ namespace
 	{
 		return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 	}
+
+	template<typename T>
+	void launch_stream_gemm(hipStream_t stream, const GemmArgs &g)
+	{
+		typedef StreamGemmConfig Cfg;
+		constexpr int STAGES = (sizeof(T) == 2) ? 8 : 7; /* the fp32 slabs are twice as large */
+		constexpr int LDS = Cfg::lds_bytes<T>(STAGES);
+		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
+		auto kernel = kernel_gemm_stream_nt<T, STAGES>;
+		static bool configured = false; /* per instantiation; the attribute belongs to the function, setting it twice is harmless */
+		if (!configured)
+		{
+			MLHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
+			configured = true;
+		}
+		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, Cfg::BN);
+		const int total_units = g.batch * tiles_m;
+		const int compute_units = device_compute_units();
+		int groups = compute_units / n_tiles;
+		if (groups >= 8)
+			groups -= groups % 8; /* keeps the grid a multiple of 8 * n_tiles so that the column slices of a group share an XCD */
+		if (groups < 1)
+			groups = 1;
+		if (groups > total_units)
+			groups = total_units;
+		const int units_per_group = ceil_div(total_units, groups);
+		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(Cfg::THREADS), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
+				reinterpret_cast<T*>(g.D), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group);
+	}
 }
 
 namespace mlhip
@@ -96,6 +126,20 @@ namespace mlhip
 		const size_t k_bytes = static_cast<size_t>(g.K) * esize;
 		const bool fast = nt && g.K > 0 && (k_bytes % 16 == 0) && aligned_to(g.A, 16) && aligned_to(g.B, 16)
 				&& ((g.stride_a * esize) % 16 == 0) && ((g.stride_b * esize) % 16 == 0);
+
+		/* The Winograd product (plain store, 512-byte rows of K, enough rows to fill the chip) takes the persistent streaming kernel. */
+		const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR);
+		if (fast && plain && k_bytes == 512 && (g.dtype == DTYPE_FLOAT16 || g.dtype == DTYPE_FLOAT32) && (g.N * esize) % 16 == 0
+				&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0) && (g.stride_a != 0 || g.batch == 1)
+				&& static_cast<size_t>(g.batch) * ceil_div(g.M, 128) >= 256)
+		{
+			if (g.dtype == DTYPE_FLOAT16)
+				launch_stream_gemm<half_t>(stream, g);
+			else
+				launch_stream_gemm<float>(stream, g);
+			MLHIP_CHECK(hipGetLastError());
+			return;
+		}
 
 		const int out_size = (g.dtype == DTYPE_INT8) ? 4 : esize;
 		const bool vectorized = (g.N % 4 == 0) && aligned_to(g.D, 4 * out_size) && aligned_to(g.C, 4 * out_size) && aligned_to(g.bias, 4 * esize)

@@ -104,6 +104,15 @@ namespace
 
 namespace mlhip
 {
+	int device_compute_units()
+	{
+		int device = 0;
+		MLHIP_CHECK(hipGetDevice(&device));
+		const std::vector<hipDeviceProp_t> &props = device_properties();
+		if (device < 0 || device >= static_cast<int>(props.size()))
+			fail_runtime("HIP backend: no current device");
+		return props[device].multiProcessorCount;
+	}
 	void* get_workspace(mlContext_t context, size_t bytes)
 	{
 		Context *ctx = get(context);

@@ -46,6 +46,29 @@ def test_gemm_batched_nt(ctx, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("shape", [(36, 1000, 256), (36, 1027, 200), (300, 128, 64), (1, 33001, 128), (36, 900, 8), (7, 5000, 384), (257, 1, 256)])
+def test_gemm_batched_nt_streaming_shapes(ctx, dtype, shape):
+    """Rows of K of exactly 512 bytes (256 halfs / 128 floats) and at least 256 row blocks: the shapes of the Winograd product in the
+    benchmark networks, which take the persistent streaming kernel. Ragged last row block, ragged and tiny N, more column slices than
+    two, runs of row blocks that cross from one matrix into the next, one-row matrices."""
+    bt, M, N = shape
+    K = 256 if dtype == "float16" else 128
+    rng = np.random.default_rng(sum(shape))
+    A = random_tensor(rng, (bt, M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (bt, N, K), dtype, 0.5)
+    dC = ml.Tensor((bt, M, N), dtype)
+    dC.setall(ctx, float("nan"))
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.0, 0.0)
+    got = dC.copyToHost(ctx)
+    assert np.isfinite(O.as_float(got)).all()
+    assert max_abs_rel(got, O.gemm(A, Bm)) <= TOL[dtype]
+    # shared B operand (rank 2) through the same kernel
+    dC.setall(ctx, float("nan"))
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm[0]), 1.0, 0.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm[0])) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_gemm_batched_broadcast_and_beta(ctx, dtype):
     rng = np.random.default_rng(5)
     A = random_tensor(rng, (4, 50, 24), dtype)
