@@ -6,9 +6,14 @@ batch of 1024 positions already resident in HBM: stem 3x3 conv 32->256, 40 3x3 c
 36 batched GEMMs on MFMA, output transform with bias + residual + ReLU), 1x1 policy head. Prints ONE JSON line:
 
   value        positions / second over the timed steps (wall clock between two stream synchronisations)
-  roofline     the 36-way batched Winograd GEMM kernel against the dense fp16 MFMA peak: executed flops of one launch
-               (2 * 36 * tiles * Cin * Cout) divided by the kernel's average duration, taken with HIP events recorded on the context's
-               stream around every launch in a second, instrumented run of the same steps
+  roofline     the dominant kernel, the 36-way batched Winograd GEMM of the 40 block convolutions. With N = K = 256 it has 127 flop per
+               byte, below the chip's ridge of ~312 flop/byte, so HBM bounds it: `achieved` = algorithmic bytes of one launch
+               (s * 36 * (T*K + N*K + T*N)) / average launch duration, against 8 TB/s. Durations come from HIP events recorded on the
+               context's stream around every launch in a second, instrumented run of the same steps. `traffic` = HBM bytes of one
+               launch from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what it reads for a copy kernel of known size);
+               the figure and the commands that produced it are in profiles/.
+  gemm_mfma    the same launches against the dense fp16 MFMA peak (executed flops 2 * 36 * T * K * N per launch)
+  transforms   input / output transform of the block convolutions: algorithmic bytes / average duration against 8 TB/s
   cpu_baseline the same network on a bounded number of positions on the host's cores: the reference's own CPU backend compiled from
                its sources (kind "reference", one thread, as the reference runs) when that library is present, otherwise this
                repository's C restatement (kind "port")
@@ -23,13 +28,19 @@ import numpy as np
 
 sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
-PEAK_FP16_MFMA_TFLOPS = 2500.0  # MI355X dense fp16 matrix peak
+PEAK_MFMA_TFLOPS = {"float16": 2500.0, "float32": 157.3}  # MI355X dense matrix peaks
 PEAK_HBM_GBS = 8000.0
 
 CONFIGS = {
     # name: (batch, board, input planes, channels, blocks, dtype, seed)
     "cfg2_resnet20x256_fp16_b1024": (1024, 15, 32, 256, 20, "float16", 1),
     "cfg1_resnet10x128_fp32_b256": (256, 15, 32, 128, 10, "float32", 0),
+}
+
+# HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each counter
+# scaled by its reading for a 256 MiB copy kernel in the same run. Source: profiles/gemm_stream_cfg2_hbm_traffic.md
+MEASURED_GEMM_TRAFFIC_BYTES = {
+    "cfg2_resnet20x256_fp16_b1024": None,
 }
 
 
@@ -62,14 +73,29 @@ def run_cpu_baseline(params_storage, x_storage, blocks, budget_seconds):
             "sample": "%d positions of the same network and inputs, one forward pass, %.1f s" % (positions, t)}
 
 
+def copy_calibration(ml, ctx):
+    """One copy kernel of known size (256 MiB read, 256 MiB written) so that a counter run can be scaled against it."""
+    n = 128 * 1024 * 1024
+    src = ml.Tensor((n,), "float16")
+    dst = ml.Tensor((n,), "float16")
+    src.zeroall(ctx)
+    dst.zeroall(ctx)
+    ml.addTensors(ctx, 1.0, src, 0.0, None, 0.0, None, 0.0, dst)  # y = 1 * x: one read and one write of every byte
+    ctx.synchronize()
+    src.free()
+    dst.free()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg2_resnet20x256_fp16_b1024", choices=sorted(CONFIGS))
-    ap.add_argument("--chunk", type=int, default=0, help="positions per cache-resident sub-batch (0 = library default)")
+    ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch one 256 MiB copy kernel (kernel_axpy3) for scaling hardware counters")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -87,6 +113,8 @@ def main():
     x = make_input(seed, batch, board, planes)
 
     ctx = ml.Context(0)
+    if args.copy_calibration:
+        copy_calibration(ml, ctx)
     net = ResNet(ctx, batch, board, planes, channels, blocks, dtype, params, to_storage, chunk=chunk)
     net.setInput(to_storage(x))
 
@@ -109,19 +137,27 @@ def main():
     kernels = timer.summary()
     ml.set_kernel_timer(None)
 
-    tiles_per_launch = net.chunk * ((board + 3) // 4) ** 2
-    gemm_flops = 2.0 * 36 * tiles_per_launch * channels * channels  # the 40 block convolutions (Cin = Cout = channels)
-    # the stem launch has Cin = planes: average flops per launch over the launches actually timed
-    launches_per_pass = (batch + net.chunk - 1) // net.chunk
-    flops_per_launch = (2 * blocks * gemm_flops + 2.0 * 36 * tiles_per_launch * planes * channels) / (2 * blocks + 1)
-    n_gemm, t_gemm = kernels.get("gemm_batched_v2", (0, float("nan")))
-    achieved = flops_per_launch / t_gemm / 1e12
+    def timed(entry, labels):
+        count = sum(kernels.get(entry + "@" + l, (0, 0.0))[0] for l in labels)
+        total = sum(kernels.get(entry + "@" + l, (0, 0.0))[0] * kernels.get(entry + "@" + l, (0, 0.0))[1] for l in labels)
+        return count, (total / count if count else float("nan"))
+
     esize = 2 if dtype == "float16" else 4
-    n_in, t_in = kernels.get("winograd_input_transform", (0, float("nan")))
-    n_out, t_out = kernels.get("winograd_output_transform", (0, float("nan")))
+    tiles = net.chunk * ((board + 3) // 4) ** 2  # T of one launch
     pix = net.chunk * board * board
-    in_bytes = esize * (pix * channels + 36 * tiles_per_launch * channels)
-    out_bytes = esize * (36 * tiles_per_launch * channels + 2 * pix * channels)  # matrices + y, + residual on every second layer
+    block_labels = ("block_conv1", "block_conv2")
+    # 36 batched GEMMs of the block convolutions (Cin = Cout = channels)
+    n_gemm, t_gemm = timed("gemm_batched_v2", block_labels)
+    gemm_flops = 2.0 * 36 * tiles * channels * channels
+    gemm_bytes = esize * 36 * (tiles * channels + channels * channels + tiles * channels)
+    gemm_gbs = gemm_bytes / t_gemm / 1e9
+    gemm_tflops = gemm_flops / t_gemm / 1e12
+    # transforms of the block convolutions; the residual is read by every second output transform
+    n_in, t_in = timed("winograd_input_transform", block_labels)
+    n_out, t_out = timed("winograd_output_transform", block_labels)
+    in_bytes = esize * (pix * channels + 36 * tiles * channels)
+    out_bytes = esize * (36 * tiles * channels + pix * channels + 0.5 * pix * channels + channels)
+    kernel_name = "kernel_gemm_stream_nt" if channels * esize == 512 else "kernel_gemm_nt"
     result = {
         "metric": "positions/sec at batch 1024 (20x256 res-net fp16); % MFMA peak in conv GEMMs" if args.config.startswith("cfg2")
         else "positions/sec (%s)" % args.config,
@@ -129,13 +165,20 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16" if dtype == "float16" else "f32",
         "data": "synthetic (Bernoulli(0.3) input planes, He-normal weights, N(0,0.01) biases, seed %d)" % seed,
         "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
-                   "cache_resident_chunk": net.chunk, "launches_per_pass_per_layer": launches_per_pass},
+                   "positions_per_launch": net.chunk},
         "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_FP16_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_FP16_MFMA_TFLOPS, "traffic": None, "kernel": "kernel_gemm_nt (36 batched Winograd GEMMs)",
-                     "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6},
-        "transforms": {"input": {"avg_launch_us": t_in * 1e6, "gbs": in_bytes / t_in / 1e9, "frac_hbm": in_bytes / t_in / 1e9 / PEAK_HBM_GBS},
-                       "output": {"avg_launch_us": t_out * 1e6, "gbs": out_bytes / t_out / 1e9, "frac_hbm": out_bytes / t_out / 1e9 / PEAK_HBM_GBS}},
+        "roofline": {"bound": "hbm", "achieved": gemm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gemm_gbs / PEAK_HBM_GBS,
+                     "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
+                     "kernel": "%s (36 batched Winograd GEMMs, M=%d N=K=%d)" % (kernel_name, tiles, channels),
+                     "algorithmic_bytes": gemm_bytes, "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6},
+        "gemm_mfma": {"achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s", "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype],
+                      "flops_per_launch": gemm_flops,
+                      "hbm_limited_ceiling_frac": min(1.0, gemm_flops / gemm_bytes * PEAK_HBM_GBS * 1e9 / (PEAK_MFMA_TFLOPS[dtype] * 1e12))},
+        "transforms": {"input": {"kernel": "kernel_input_transform_4x4_3x3", "launches_timed": n_in, "avg_launch_us": t_in * 1e6,
+                                 "algorithmic_bytes": in_bytes, "gbs": in_bytes / t_in / 1e9, "frac_hbm": in_bytes / t_in / 1e9 / PEAK_HBM_GBS},
+                       "output": {"kernel": "kernel_output_transform_4x4_3x3", "launches_timed": n_out, "avg_launch_us": t_out * 1e6,
+                                  "algorithmic_bytes": out_bytes, "gbs": out_bytes / t_out / 1e9,
+                                  "frac_hbm": out_bytes / t_out / 1e9 / PEAK_HBM_GBS}},
     }
     if args.cpu_seconds > 0:
         params_storage = [(to_storage(w), to_storage(b)) for (w, b) in params]

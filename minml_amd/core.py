@@ -231,6 +231,8 @@ class KernelTimer:
         function(*args)
         end = Event(self.context)
         self.records.setdefault(name, []).append((start, end))
+        if _TIMER_LABEL is not None:
+            self.records.setdefault(name + "@" + _TIMER_LABEL, []).append((start, end))
 
     def summary(self):
         self.context.synchronize()
@@ -238,19 +240,28 @@ class KernelTimer:
         for name, pairs in self.records.items():
             total = sum(Event.getElapsedTime(s, e) for s, e in pairs)
             result[name] = (len(pairs), total / len(pairs))
-            for s, e in pairs:
-                s.destroy()
-                e.destroy()
+        for name, pairs in self.records.items():
+            if "@" not in name:  # labelled entries share their events with the unlabelled ones
+                for s, e in pairs:
+                    s.destroy()
+                    e.destroy()
         self.records = {}
         return result
 
 
 _TIMER = None
+_TIMER_LABEL = None
 
 
 def set_kernel_timer(timer):
     global _TIMER
     _TIMER = timer
+
+
+def set_timer_label(label):
+    """While a kernel timer is installed, launches are also recorded under "<entry point>@<label>" (None switches this off)."""
+    global _TIMER_LABEL
+    _TIMER_LABEL = label
 
 
 def _launch(name, *args):

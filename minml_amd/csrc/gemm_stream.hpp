@@ -242,15 +242,8 @@ namespace mlhip
 						const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
 						const int m = m_first + 32 * i + row;
 						const int n = n0 + wave_n * 64 + col;
-						if (m < M && n + ELEMS_PER_16B <= N)
+						if (m < M && n < N) /* N is a multiple of the 16-byte vector (checked by the launcher), so a vector is all in or all out */
 							*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n) = v;
-						else if (m < M && n < N)
-						{ /* ragged right edge: element by element */
-							const T *src = reinterpret_cast<const T*>(slab + row * SLAB_STRIDE) + col;
-							for (int e = 0; e < ELEMS_PER_16B; e++)
-								if (n + e < N)
-									c_base[static_cast<size_t>(m) * N + n + e] = src[e];
-						}
 					}
 					__builtin_amdgcn_s_waitcnt(0xc07f);
 					__builtin_amdgcn_wave_barrier();
@@ -260,6 +253,10 @@ namespace mlhip
 			for (int g = 0; g < DISTANCE; g++)
 				if (g < run_stages)
 					request_stage(g);
+			/* The B operand must have arrived before the first multiply. Waiting for everything here (B and the first stages, whose
+			 * latencies overlap) costs one memory latency per run and leaves the compiler with no outstanding register loads to track:
+			 * otherwise it guards every multiply in the loop below with a full vmcnt(0), which drains the ring at every stage. */
+			wait_vmcnt<0>();
 			clear_accumulators();
 
 			uint4_t frags[2][4][2];

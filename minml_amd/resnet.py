@@ -6,8 +6,9 @@ ReLU); policy head 1x1 conv to one channel (+bias, linear). Layers run in insert
 to the largest request, as the reference's Graph does (src/graph/Graph.cpp:241-248,578-587).
 
 `chunk` splits the batch into sub-batches that are pushed through the whole network one after the other. The layer entry points are
-batch-size agnostic, so this changes nothing in the results; it keeps the Winograd matrices of a sub-batch (2 x 36 x 16 x chunk x C
-elements) inside the 256 MB last-level cache between the transform and GEMM kernels instead of streaming them through HBM.
+batch-size agnostic, so this changes nothing in the results; it bounds the workspace (2 x 36 x 16 x chunk x C elements). Measured on
+MI355X, sub-batches small enough for the Winograd matrices to stay in the 256 MB last-level cache between the transform and GEMM
+kernels were not faster than streaming the whole batch through HBM, so the default is the whole batch.
 """
 import numpy as np
 
@@ -16,7 +17,7 @@ from . import core as ml
 from .conv2d import Conv2D
 
 
-# positions per sub-batch pushed through the whole network at once, by storage type (measured choice; see ResNet docstring)
+# positions per sub-batch pushed through the whole network at once, by storage type (measured choice: the whole benchmark batch)
 DEFAULT_CHUNK = {"float16": 1024, "float32": 256}
 
 
@@ -81,12 +82,17 @@ class ResNet:
             n = min(self.chunk, self.batch - start)
             x = self._view_batch(self.input, start, n)
             a, b, c = (self._view_batch(t, 0, n) for t in self.act)
+            ml.set_timer_label("stem")
             self.layers[0].forward([x], a, self.workspace)
             for blk in range(self.blocks):
+                ml.set_timer_label("block_conv1")
                 self.layers[1 + 2 * blk].forward([a], b, self.workspace)
+                ml.set_timer_label("block_conv2")
                 self.layers[2 + 2 * blk].forward([b, a], c, self.workspace)
                 a, c = c, a
+            ml.set_timer_label("head")
             self.layers[-1].forward([a], self._view_batch(self.output, start, n), self.workspace)
+            ml.set_timer_label(None)
         return self.output
 
     def trunk_output(self):
