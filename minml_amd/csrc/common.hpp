@@ -62,6 +62,8 @@ namespace mlhip
 	void* get_workspace(mlContext_t context, size_t bytes);
 	/* number of compute units of the current device (cached per device) */
 	int device_compute_units();
+	/* opts a kernel in to `bytes` of dynamic LDS (more than the 64 KB default) on the current device; remembered per device and kernel */
+	void ensure_dynamic_lds(const void *kernel, int bytes);
 
 	inline int size_of(mlDataType_t dtype)
 	{

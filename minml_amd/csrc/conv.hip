@@ -15,6 +15,7 @@
 #include "gemm_core.hpp"
 #include "epilogues.hpp"
 #include "gemm_launch.hpp"
+#include "gemm_dma.hpp"
 
 #include <cstring>
 
@@ -146,20 +147,8 @@ namespace
 		const size_t c_bytes = static_cast<size_t>(filters_in) * sizeof(T);
 		const size_t k_bytes = c_bytes * kernel_h * kernel_w;
 		const bool fast = (c_bytes % 16 == 0) && aligned16(input) && aligned16(weights) && k_bytes <= 0x7fffffffu;
-		if (fast)
+		const auto make_epilogue = [&]()
 		{
-			typedef TileConfig<128, 128, 64, 2, 2> Cfg;
-			Im2RowRows<T> a_loader;
-			a_loader.base = reinterpret_cast<const T*>(input);
-			a_loader.rows = M;
-			a_loader.height = height;
-			a_loader.width = width;
-			a_loader.kernel_h = kernel_h;
-			a_loader.kernel_w = kernel_w;
-			a_loader.c_bytes = static_cast<int>(c_bytes);
-			a_loader.k_bytes = static_cast<int>(k_bytes);
-			a_loader.fill = 0u;
-
 			FloatEpilogue<T> ep;
 			ep.D = reinterpret_cast<T*>(output);
 			ep.C = reinterpret_cast<const T*>(add);
@@ -172,6 +161,36 @@ namespace
 			const size_t vbytes = 4 * sizeof(T);
 			ep.vectorized = (filters_out % 4 == 0) && (reinterpret_cast<uintptr_t>(output) % vbytes == 0) && (reinterpret_cast<uintptr_t>(add) % vbytes == 0)
 					&& (reinterpret_cast<uintptr_t>(bias) % vbytes == 0);
+			return ep;
+		};
+		if (fast && c_bytes % 128 == 0)
+		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */
+			Im2RowDmaRows a_loader;
+			a_loader.base = reinterpret_cast<const uint8_t*>(input);
+			a_loader.rows = M;
+			a_loader.height = height;
+			a_loader.width = width;
+			a_loader.kernel_h = kernel_h;
+			a_loader.kernel_w = kernel_w;
+			a_loader.c_bytes = static_cast<int>(c_bytes);
+			a_loader.fill = 0;
+			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(weights), filters_out, static_cast<int>(k_bytes) };
+			launch_gemm_dma<T>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, make_epilogue());
+		}
+		else if (fast)
+		{
+			typedef TileConfig<128, 128, 64, 2, 2> Cfg;
+			Im2RowRows<T> a_loader;
+			a_loader.base = reinterpret_cast<const T*>(input);
+			a_loader.rows = M;
+			a_loader.height = height;
+			a_loader.width = width;
+			a_loader.kernel_h = kernel_h;
+			a_loader.kernel_w = kernel_w;
+			a_loader.c_bytes = static_cast<int>(c_bytes);
+			a_loader.k_bytes = static_cast<int>(k_bytes);
+			a_loader.fill = 0u;
+			const FloatEpilogue<T> ep = make_epilogue();
 
 			const int tiles_m = ceil_div(M, Cfg::BM), tiles_n = ceil_div(filters_out, Cfg::BN);
 			const dim3 grid(static_cast<unsigned int>(tiles_m) * tiles_n);

@@ -40,6 +40,62 @@ namespace mlhip
 				}
 				return x;
 			}
+			/*
+			 * Split form for kernels that want the side inputs in flight early (only when `vectorized`): the per-column constants of 4
+			 * consecutive n, the per-element side input (beta * C) of one group, and the tail that consumes both. Same arithmetic and
+			 * order as operator().
+			 */
+			struct Column
+			{
+					float bias[4];
+			};
+			struct Extra
+			{
+					Vec<T, 4> c;
+			};
+			__device__ __forceinline__ Column load_column(int n) const
+			{
+				Column col;
+				Vec<T, 4> b;
+				b.zero();
+				if (bias != nullptr)
+					b.load(bias + n);
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					col.bias[e] = b.v[e];
+				return col;
+			}
+			__device__ __forceinline__ Extra load_extra(int m, int n) const
+			{
+				Extra x;
+				x.c.zero();
+				if (beta != 0.0f)
+					x.c.load(C + static_cast<size_t>(m) * row_stride + n);
+				return x;
+			}
+			__device__ __forceinline__ void apply(int m, int n, const float (&acc)[4], const Column &col, const Extra &x) const
+			{
+				Vec<T, 4> out;
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					out.v[e] = acc[e] * alpha;
+				if (bias != nullptr)
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] += col.bias[e];
+				}
+				if (beta != 0.0f)
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] += beta * x.c.v[e];
+				}
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					out.v[e] = finish(out.v[e]);
+				out.store(D + static_cast<size_t>(m) * row_stride + n);
+			}
 			__device__ __forceinline__ void operator()(int m, int n, const float (&acc)[4]) const
 			{
 				if (n >= N)
@@ -98,6 +154,24 @@ namespace mlhip
 			bool vectorized;
 			static constexpr bool has_c = false;
 
+			struct Column
+			{
+			};
+			struct Extra
+			{
+			};
+			__device__ __forceinline__ Column load_column(int) const
+			{
+				return Column { };
+			}
+			__device__ __forceinline__ Extra load_extra(int, int) const
+			{
+				return Extra { };
+			}
+			__device__ __forceinline__ void apply(int m, int n, const int (&acc)[4], const Column&, const Extra&) const
+			{
+				*reinterpret_cast<int4_t*>(D + static_cast<size_t>(m) * row_stride + n) = int4_t { acc[0], acc[1], acc[2], acc[3] };
+			}
 			__device__ __forceinline__ void operator()(int m, int n, const int (&acc)[4]) const
 			{
 				if (n >= N)
@@ -176,6 +250,56 @@ namespace mlhip
 			bool vectorized; /* N % 4 == 0 and all pointers 4-element aligned */
 			static constexpr bool has_c = false;
 
+			struct Column
+			{
+					float4_t scales, bias;
+			};
+			struct Extra
+			{
+					uint32_t packed;
+			};
+			__device__ __forceinline__ Column load_column(int n) const
+			{
+				Column col;
+				col.scales = *reinterpret_cast<const float4_t*>(scales + n);
+				col.bias = *reinterpret_cast<const float4_t*>(bias + n);
+				return col;
+			}
+			__device__ __forceinline__ Extra load_extra(int m, int n) const
+			{
+				Extra x;
+				x.packed = 0;
+				if (ext != nullptr)
+					x.packed = *reinterpret_cast<const uint32_t*>(ext + static_cast<size_t>(m) * row_stride + n);
+				return x;
+			}
+			__device__ __forceinline__ void apply(int m, int n, const int (&acc)[4], const Column &col, const Extra &x) const
+			{
+				const size_t offset = static_cast<size_t>(m) * row_stride + n;
+				float vals[4];
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+				{
+					const int ext_val = static_cast<int>(static_cast<int8_t>((x.packed >> (8 * e)) & 0xffu));
+					vals[e] = requant_value(acc[e], col.scales[e], col.bias[e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+				}
+				if constexpr (sizeof(OutT) == 1)
+				{
+					uint32_t packed = 0;
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						packed |= (static_cast<uint32_t>(quantize_to_int8(vals[e], inv_scale, inv_shift)) & 0xffu) << (8 * e);
+					*reinterpret_cast<uint32_t*>(D + offset) = packed;
+				}
+				else
+				{
+					Vec<OutT, 4> out;
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] = vals[e];
+					out.store(D + offset);
+				}
+			}
 			__device__ __forceinline__ void operator()(int m, int n, const int (&acc)[4]) const
 			{
 				if (n >= N)

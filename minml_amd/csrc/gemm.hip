@@ -17,6 +17,7 @@
 #include "epilogues.hpp"
 #include "gemm_launch.hpp"
 #include "gemm_stream.hpp"
+#include "gemm_dma.hpp"
 
 namespace
 {
@@ -149,6 +150,11 @@ namespace mlhip
 		const size_t a_row = g.transpose_a ? 1 : g.K, a_col = g.transpose_a ? g.M : 1;
 		const size_t b_row = g.transpose_b ? g.K : 1, b_col = g.transpose_b ? 1 : g.N;
 
+		/* K rows that are whole 128-byte chunks take the direct-to-LDS engine */
+		const bool dma = fast && (k_bytes % 128 == 0) && k_bytes <= 0x7fffffffu;
+		const DenseDmaRows dma_a { reinterpret_cast<const uint8_t*>(g.A), g.M, static_cast<int>(k_bytes) };
+		const DenseDmaRows dma_b { reinterpret_cast<const uint8_t*>(g.B), g.N, static_cast<int>(k_bytes) };
+
 		typedef TileConfig<128, 128, 64, 2, 2> Cfg;
 		const int tiles_m = ceil_div(g.M, Cfg::BM), tiles_n = ceil_div(g.N, Cfg::BN);
 		const dim3 fast_grid(static_cast<unsigned int>(tiles_m) * tiles_n, g.batch);
@@ -170,7 +176,10 @@ namespace mlhip
 				ep.beta = g.beta;
 				ep.act = g.act;
 				ep.vectorized = vectorized;
-				if (fast)
+				if (dma)
+					launch_gemm_dma<half_t>(stream, dma_a, dma_b, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a * esize, g.stride_b * esize,
+							g.stride_c, ep);
+				else if (fast)
 					hipLaunchKernelGGL((kernel_gemm_nt<half_t, Cfg, FloatEpilogue<half_t>>), fast_grid, dim3(Cfg::THREADS), 0, stream,
 							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
 							g.stride_b, g.stride_c, ep, tiles_n);
@@ -192,7 +201,10 @@ namespace mlhip
 				ep.beta = g.beta;
 				ep.act = g.act;
 				ep.vectorized = vectorized;
-				if (fast)
+				if (dma)
+					launch_gemm_dma<float>(stream, dma_a, dma_b, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a * esize, g.stride_b * esize,
+							g.stride_c, ep);
+				else if (fast)
 					hipLaunchKernelGGL((kernel_gemm_nt<float, Cfg, FloatEpilogue<float>>), fast_grid, dim3(Cfg::THREADS), 0, stream,
 							reinterpret_cast<const float*>(g.A), reinterpret_cast<const float*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
 							g.stride_b, g.stride_c, ep, tiles_n);
@@ -210,7 +222,10 @@ namespace mlhip
 				ep.N = g.N;
 				ep.row_stride = g.N;
 				ep.vectorized = vectorized;
-				if (fast)
+				if (dma)
+					launch_gemm_dma<int8_t>(stream, dma_a, dma_b, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a * esize, g.stride_b * esize,
+							g.stride_c, ep);
+				else if (fast)
 					hipLaunchKernelGGL((kernel_gemm_nt<int8_t, Cfg, Int32Epilogue>), fast_grid, dim3(Cfg::THREADS), 0, stream,
 							reinterpret_cast<const int8_t*>(g.A), reinterpret_cast<const int8_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
 							g.stride_b, g.stride_c, ep, tiles_n);

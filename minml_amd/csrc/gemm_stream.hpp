@@ -134,7 +134,7 @@ namespace mlhip
 		{
 			const int row = (wave + 4 * i) * 8 + (lane >> 3);
 			load_row[i] = row;
-			load_chunk_bytes[i] = ((lane & 7) ^ ((row + (row >> 3)) & 7)) * 16;
+			load_chunk_bytes[i] = ((lane & 7) ^ ((row >> 1) & 7)) * 16;
 		}
 		/* fragment geometry: lane l supplies row l % 32 and the 16-byte half l / 32 of each 32-byte k step */
 		const int frag_row = lane & 31;
@@ -145,7 +145,7 @@ namespace mlhip
 		{
 			const int row = wave_m * 64 + i * 32 + frag_row;
 			frag_offset[i] = row * Cfg::STAGE_K_BYTES;
-			frag_swizzle[i] = (row + (row >> 3)) & 7;
+			frag_swizzle[i] = (row >> 1) & 7;
 		}
 
 		int unit = unit_begin;

@@ -15,6 +15,7 @@
 #include "common.hpp"
 #include "gemm_core.hpp"
 #include "epilogues.hpp"
+#include "gemm_dma.hpp"
 
 #include <cmath>
 
@@ -170,7 +171,21 @@ namespace
 		const size_t k_bytes = static_cast<size_t>(filters_in) * kernel_h * kernel_w;
 		const bool zero_fits = (input_zero >= -128 && input_zero <= 127) || (kernel_h == 1 && kernel_w == 1);
 		const bool fast = (filters_in % 16 == 0) && aligned_to(input, 16) && aligned_to(weights, 16) && k_bytes <= 0x7fffffffu && zero_fits;
-		if (fast)
+		if (fast && filters_in % 128 == 0)
+		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */
+			Im2RowDmaRows a_loader;
+			a_loader.base = reinterpret_cast<const uint8_t*>(input);
+			a_loader.rows = M;
+			a_loader.height = height;
+			a_loader.width = width;
+			a_loader.kernel_h = kernel_h;
+			a_loader.kernel_w = kernel_w;
+			a_loader.c_bytes = filters_in;
+			a_loader.fill = input_zero & 0xff; /* a 1x1 kernel never pads, so an out-of-range zero point is harmless there */
+			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(weights), filters_out, static_cast<int>(k_bytes) };
+			launch_gemm_dma<int8_t>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, ep);
+		}
+		else if (fast)
 		{
 			typedef TileConfig<128, 128, 64, 2, 2> Cfg;
 			Im2RowRows<int8_t> a_loader;

@@ -6,8 +6,10 @@
 
 #include <cstring>
 #include <mutex>
+#include <set>
 #include <sstream>
 #include <string>
+#include <utility>
 #include <vector>
 
 namespace
@@ -112,6 +114,16 @@ namespace mlhip
 		if (device < 0 || device >= static_cast<int>(props.size()))
 			fail_runtime("HIP backend: no current device");
 		return props[device].multiProcessorCount;
+	}
+	void ensure_dynamic_lds(const void *kernel, int bytes)
+	{
+		static std::mutex guard;
+		static std::set<std::pair<int, const void*>> configured;
+		int device = 0;
+		MLHIP_CHECK(hipGetDevice(&device));
+		std::lock_guard<std::mutex> lock(guard);
+		if (configured.insert(std::make_pair(device, kernel)).second)
+			MLHIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
 	}
 	void* get_workspace(mlContext_t context, size_t bytes)
 	{
