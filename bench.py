@@ -3,7 +3,9 @@
 
 A step is one forward pass of the synthetic 20-block x 256-channel 15x15 residual network (fp16 storage, fp32 accumulation) over one
 batch of 1024 positions already resident in HBM: stem 3x3 conv 32->256, 40 3x3 convs 256->256 as Winograd F(4x4,3x3) (input transform,
-36 batched GEMMs on MFMA, output transform with bias + residual + ReLU), 1x1 policy head. Prints ONE JSON line:
+36 batched GEMMs on MFMA, output transform with bias + residual + ReLU), 1x1 policy head. By default the output transform of each 3x3
+layer and the input transform of the next run as one launch (bit-identical results; --unfused runs the reference's three calls per
+layer). Prints ONE JSON line:
 
   value        positions / second over the timed steps (wall clock between two stream synchronisations)
   roofline     the dominant kernel, the 36-way batched Winograd GEMM of the 40 block convolutions. With N = K = 256 it has 127 flop per
@@ -13,7 +15,7 @@ batch of 1024 positions already resident in HBM: stem 3x3 conv 32->256, 40 3x3 c
                launch from rocprofv3 counters (FETCH_SIZE + WRITE_SIZE, each scaled by what it reads for a copy kernel of known size);
                the figure and the commands that produced it are in profiles/.
   gemm_mfma    the same launches against the dense fp16 MFMA peak (executed flops 2 * 36 * T * K * N per launch)
-  transforms   input / output transform of the block convolutions: algorithmic bytes / average duration against 8 TB/s
+  transforms   the transform launches of the block convolutions: algorithmic bytes / average duration against 8 TB/s
   cpu_baseline the same network on a bounded number of positions on the host's cores: the reference's own CPU backend compiled from
                its sources (kind "reference", one thread, as the reference runs) when that library is present, otherwise this
                repository's C restatement (kind "port")
@@ -95,6 +97,7 @@ def main():
     ap.add_argument("--config", default="cfg2_resnet20x256_fp16_b1024", choices=sorted(CONFIGS))
     ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
+    ap.add_argument("--unfused", action="store_true", help="run every layer as the reference's three calls (no cross-layer transform fusion)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB copy kernel (kernel_axpy3) for scaling hardware counters")
     args = ap.parse_args()
@@ -116,7 +119,7 @@ def main():
     ctx = ml.Context(0)
     if args.copy_calibration:
         copy_calibration(ml, ctx)
-    net = ResNet(ctx, batch, board, planes, channels, blocks, dtype, params, to_storage, chunk=chunk)
+    net = ResNet(ctx, batch, board, planes, channels, blocks, dtype, params, to_storage, chunk=chunk, fused=not args.unfused)
     net.setInput(to_storage(x))
 
     for _ in range(args.warmup):
@@ -153,11 +156,22 @@ def main():
     gemm_bytes = esize * 36 * (tiles * channels + channels * channels + tiles * channels)
     gemm_gbs = gemm_bytes / t_gemm / 1e9
     gemm_tflops = gemm_flops / t_gemm / 1e12
-    # transforms of the block convolutions; the residual is read by every second output transform
-    n_in, t_in = timed("winograd_input_transform", block_labels)
-    n_out, t_out = timed("winograd_output_transform", block_labels)
-    in_bytes = esize * (pix * channels + 36 * tiles * channels)
-    out_bytes = esize * (36 * tiles * channels + pix * channels + 0.5 * pix * channels + channels)
+    # transforms of the block convolutions. Fused mode: inside a residual block one launch does the first convolution's output transform
+    # and the second one's input transform (nothing else read or written); block boundaries use the two stand-alone transforms.
+    mat_bytes = esize * 36 * tiles * channels
+    act_bytes = esize * pix * channels
+    transforms = {}
+    for entry, kernel, label, nbytes in (
+            ("winograd_output_input_transform", "kernel_output_input_transform_4x4_3x3", "block_conv1", 2 * mat_bytes),
+            ("winograd_output_input_transform", "kernel_output_input_transform_4x4_3x3 (+residual, y written)", "block_conv2", 2 * mat_bytes + 2 * act_bytes),
+            ("winograd_input_transform", "kernel_input_transform_4x4_3x3", "block_conv1", mat_bytes + act_bytes),
+            ("winograd_input_transform", "kernel_input_transform_4x4_3x3", "block_conv2", mat_bytes + act_bytes),
+            ("winograd_output_transform", "kernel_output_transform_4x4_3x3", "block_conv1", mat_bytes + act_bytes),
+            ("winograd_output_transform", "kernel_output_transform_4x4_3x3 (+residual)", "block_conv2", mat_bytes + 2 * act_bytes)):
+        n_t, t_t = timed(entry, (label,))
+        if n_t:
+            transforms["%s@%s" % (entry, label)] = {"kernel": kernel, "launches_timed": n_t, "avg_launch_us": t_t * 1e6, "algorithmic_bytes": nbytes,
+                                                   "gbs": nbytes / t_t / 1e9, "frac_hbm": nbytes / t_t / 1e9 / PEAK_HBM_GBS}
     kernel_name = "kernel_gemm_stream_nt" if channels * esize == 512 else "kernel_gemm_nt"
     result = {
         "metric": "positions/sec at batch 1024 (20x256 res-net fp16); % MFMA peak in conv GEMMs" if args.config.startswith("cfg2")
@@ -166,7 +180,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16" if dtype == "float16" else "f32",
         "data": "synthetic (Bernoulli(0.3) input planes, He-normal weights, N(0,0.01) biases, seed %d)" % seed,
         "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
-                   "positions_per_launch": net.chunk},
+                   "positions_per_launch": net.chunk, "cross_layer_transform_fusion": not args.unfused},
         "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
         "roofline": {"bound": "hbm", "achieved": gemm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gemm_gbs / PEAK_HBM_GBS,
                      "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
@@ -175,11 +189,7 @@ def main():
         "gemm_mfma": {"achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s", "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype],
                       "flops_per_launch": gemm_flops,
                       "hbm_limited_ceiling_frac": min(1.0, gemm_flops / gemm_bytes * PEAK_HBM_GBS * 1e9 / (PEAK_MFMA_TFLOPS[dtype] * 1e12))},
-        "transforms": {"input": {"kernel": "kernel_input_transform_4x4_3x3", "launches_timed": n_in, "avg_launch_us": t_in * 1e6,
-                                 "algorithmic_bytes": in_bytes, "gbs": in_bytes / t_in / 1e9, "frac_hbm": in_bytes / t_in / 1e9 / PEAK_HBM_GBS},
-                       "output": {"kernel": "kernel_output_transform_4x4_3x3", "launches_timed": n_out, "avg_launch_us": t_out * 1e6,
-                                  "algorithmic_bytes": out_bytes, "gbs": out_bytes / t_out / 1e9,
-                                  "frac_hbm": out_bytes / t_out / 1e9 / PEAK_HBM_GBS}},
+        "transforms": transforms,
     }
     if args.cpu_seconds > 0:
         params_storage = [(to_storage(w), to_storage(b)) for (w, b) in params]

@@ -106,6 +106,15 @@ extern "C"
 	void hip_winograd_input_transform(mlContext_t context, int tile_size, const mlTensor_t x, mlTensor_t matrices);
 	void hip_winograd_output_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
 			mlTensor_t y, mlActivationType_t act);
+	/*
+	 * hip_winograd_output_input_transform: hip_winograd_output_transform of one layer followed by hip_winograd_input_transform of the
+	 * next 3x3 layer on the result, in one launch; bit-identical to the two calls. `output` may be NULL when y is not needed in
+	 * memory (for channel counts that are multiples of 64; other shapes run the two transforms through `output`, which must then be
+	 * given). No counterpart in the reference, whose layers call the two transforms separately (src/layers/Conv2D.cpp:365-378): it
+	 * removes one write and one read of the activation tensor per layer from the Winograd path.
+	 */
+	void hip_winograd_output_input_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
+			mlShape_t output_shape, void *output, mlActivationType_t act, mlTensor_t next_matrices);
 
 	/* ---- GEMMs (reference: cuda_backend.h:147-154; semantics of src/backend/cpu/gemm/gemm.cpp:34-83).
 	 *      C.dtype == INT32 selects the int8 x int8 -> int32 product (src/backend/cuda/gemms.cpp:119-130). ---- */

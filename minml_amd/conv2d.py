@@ -119,18 +119,45 @@ class Conv2D:
         elif self.forward_algorithm == EXPLICIT_GEMM:
             ml.explicit_gemm_forward(ctx, x, output, self.weights, self.bias, workspace, self.activation, add)
         else:
-            if self.transformed_weights is None:
-                self.transformed_weights = ml.Tensor(get_weight_matrices_shape(self.weight_shape, self.winograd_tile_size), self.dtype,
-                                                     ctx.device_index)
-                ml.winogradWeightTransform(ctx, self.weights, self.transformed_weights, False)
-            in_shape = get_matrices_shape(self.kernel_size, self.winograd_tile_size, x.shape)
-            out_shape = get_matrices_shape(self.kernel_size, self.winograd_tile_size, output.shape)
-            input_matrices = workspace.view(in_shape)
-            output_matrices = workspace.view(out_shape, int(np.prod(in_shape)))
-            ml.winogradInputTransform(ctx, self.weight_shape, x, input_matrices)
-            ml.gemmBatched(ctx, "n", "t", output_matrices, input_matrices, self.transformed_weights, 1.0, 0.0)
-            ml.winogradOutputTransform(ctx, self.weight_shape, output_matrices, output, self.bias, add, self.activation)
+            self.winograd_input(x, workspace)
+            self.winograd_gemm(x.shape[0], workspace)
+            self.winograd_output(output, add, workspace)
         return output
+
+    # ---- the three stages of the Winograd path, separately callable so that a runner can fuse across layers -------------------
+    def _winograd_views(self, batch, workspace):
+        """(input matrices, output matrices): views at element 0 and 36*T*Cin of the workspace (Conv2D.cpp:365-367)."""
+        in_shape = get_matrices_shape(self.kernel_size, self.winograd_tile_size, (batch,) + self.input_shape[1:])
+        out_shape = get_matrices_shape(self.kernel_size, self.winograd_tile_size, (batch,) + self.output_shape[1:])
+        return workspace.view(in_shape), workspace.view(out_shape, int(np.prod(in_shape)))
+
+    def winograd_input(self, x, workspace):
+        input_matrices, _ = self._winograd_views(x.shape[0], workspace)
+        ml.winogradInputTransform(self.context, self.weight_shape, x, input_matrices)
+
+    def winograd_gemm(self, batch, workspace):
+        """36 batched products of the input matrices already in the workspace with the cached transformed weights."""
+        ctx = self.context
+        if self.transformed_weights is None:
+            self.transformed_weights = ml.Tensor(get_weight_matrices_shape(self.weight_shape, self.winograd_tile_size), self.dtype, ctx.device_index)
+            ml.winogradWeightTransform(ctx, self.weights, self.transformed_weights, False)
+        input_matrices, output_matrices = self._winograd_views(batch, workspace)
+        ml.gemmBatched(ctx, "n", "t", output_matrices, input_matrices, self.transformed_weights, 1.0, 0.0)
+
+    def winograd_output(self, output, add, workspace):
+        _, output_matrices = self._winograd_views(output.shape[0], workspace)
+        ml.winogradOutputTransform(self.context, self.weight_shape, output_matrices, output, self.bias, add, self.activation)
+
+    def winograd_output_into(self, next_layer, batch, output, add, workspace):
+        """Output transform of this layer fused with the input transform of `next_layer` (a Winograd layer on this layer's output,
+        sharing the workspace): the next layer's input matrices land at element 0, where this layer's are no longer needed.
+        `output` may be None when nothing else reads this layer's result."""
+        _, output_matrices = self._winograd_views(batch, workspace)
+        next_input, _ = next_layer._winograd_views(batch, workspace)
+        if next_input.volume() > self._winograd_views(batch, workspace)[0].volume():
+            raise ValueError("the next layer's input matrices would overlap this layer's output matrices in the workspace")
+        out_shape = (batch,) + self.output_shape[1:]
+        ml.winogradOutputInputTransform(self.context, self.weight_shape, output_matrices, out_shape, output, self.bias, add, self.activation, next_input)
 
     def _forward_int8(self, x, add, output, workspace):
         ctx = self.context

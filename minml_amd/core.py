@@ -317,6 +317,23 @@ def winogradOutputTransform(context, weight_shape, matrices, output, bias, add, 
     _launch("winograd_output_transform", context.handle, tile, matrices.desc(), _desc(bias), _desc(add), output.desc(), act_of(act))
 
 
+def winogradOutputInputTransform(context, weight_shape, matrices, output_shape, output, bias, add, act, next_matrices):
+    """Output transform of one layer fused with the input transform of the next 3x3 layer (no counterpart in the reference's math.hpp).
+    `output` may be None when y itself is not needed in memory."""
+    tile = get_winograd_tile(weight_shape, matrices.shape)
+    _require_winograd_supported(tile, weight_shape[1], matrices.dtype)
+    _require(_same_dtype(matrices, next_matrices, output, bias, add), "dtype mismatch")
+    b, h, w, c = output_shape
+    expected = (36, b * ((h + 3) // 4) * ((w + 3) // 4), c)
+    _require(matrices.shape == expected and next_matrices.shape == expected, "matrices must be [36, tiles, C]")
+    _require(output is None or output.shape == tuple(output_shape), "output must have the given shape")
+    _require(bias is None or bias.isEmpty() or bias.volume() == c, "bias must be [C]")
+    _require(add is None or add.isEmpty() or add.shape == tuple(output_shape), "add must have the output's shape")
+    _require(output is not None or c % 64 == 0, "without an output tensor the channel count must be a multiple of 64")
+    _launch("winograd_output_input_transform", context.handle, tile, matrices.desc(), _desc(bias), _desc(add), B.make_shape(output_shape), _ptr(output),
+            act_of(act), next_matrices.desc())
+
+
 def _gemm_dims(opA, A, opB, Bm):
     ta, tb = opA in "tT", opB in "tT"
     _require(opA in "ntNT" and opB in "ntNT", "op must be n or t")

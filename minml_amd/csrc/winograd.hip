@@ -360,6 +360,201 @@ namespace
 		}
 	}
 
+	/*
+	 * Output transform of one layer fused with the input transform of the next 3x3 layer:
+	 *   matrices [36][tiles][C] (+ bias, + ext) -> y [B][H][W][C] (written only if `output` is given) -> next_matrices [36][tiles][C]
+	 * One workgroup owns one image and a slice of SLICE channels: its 256 threads are 256 / (SLICE / VEC) tile lanes x SLICE / VEC
+	 * channel lanes. Phase 1 runs the output transform of the image's tiles (same arithmetic and epilogue as the stand-alone kernel) and
+	 * leaves y, rounded to the storage type as the stand-alone kernel would store it, in LDS; phase 2 reads the 6x6 windows back
+	 * (zero outside the image) and runs the input transform. Results are bit-identical to the two separate calls; what is saved is
+	 * the write and re-read of y through HBM (or only the re-read, when y is also needed as a later residual).
+	 */
+	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT>
+	__global__ __launch_bounds__(256, 2) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+			const T *ext, int act, T *__restrict__ next_matrices, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
+	{
+		typedef typename RawVec<T, VEC>::type raw_t;
+		constexpr int CHANNEL_LANES = SLICE / VEC;
+		constexpr int TILE_LANES = 256 / CHANNEL_LANES;
+		extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
+		T *image = reinterpret_cast<T*>(lds_bytes); /* [height * width + 1][SLICE]; the extra last pixel stays zero */
+
+		const unsigned int slices = channels / SLICE;
+		const unsigned int batch = blockIdx.x / slices;
+		const unsigned int slice = blockIdx.x - batch * slices;
+		const int channel_local = (threadIdx.x % CHANNEL_LANES) * VEC;
+		const unsigned int channel = slice * SLICE + channel_local;
+		const int tile_lane = threadIdx.x / CHANNEL_LANES;
+		const unsigned int tiles_per_image = tiles_h * tiles_w;
+		const unsigned int nb_of_tiles = batch_size * tiles_per_image;
+		const size_t matrix_stride = static_cast<size_t>(nb_of_tiles) * channels;
+		const int zero_pixel = height * width;
+
+		if (tile_lane == 0)
+		{
+			Vec<T, VEC> z;
+			z.zero();
+			z.store(image + zero_pixel * SLICE + channel_local);
+		}
+		Vec<T, VEC> b;
+		if (bias != nullptr)
+			b.load(bias + channel);
+		else
+			b.zero();
+
+		/* ---- phase 1: output transform into LDS (and to `output`) ---- */
+#pragma clang loop unroll(disable)
+		for (unsigned int in_image = tile_lane; in_image < tiles_per_image; in_image += TILE_LANES)
+		{
+			const unsigned int tile_idx = batch * tiles_per_image + in_image;
+			const int tile_x = in_image / tiles_w;
+			const int x0 = 4 * tile_x;
+			const int y0 = 4 * (in_image - tile_x * tiles_w);
+
+			const T *src = matrices + static_cast<size_t>(tile_idx) * channels + channel;
+			raw_t raw[6][6];
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+#pragma unroll
+				for (int col = 0; col < 6; col++)
+					raw[row][col] = *reinterpret_cast<const raw_t*>(src + static_cast<size_t>(row * 6 + col) * matrix_stride);
+
+			int pixel[4][4]; /* pixel index within the image, clamped */
+#pragma unroll
+			for (int row = 0; row < 4; row++)
+#pragma unroll
+				for (int col = 0; col < 4; col++)
+					pixel[row][col] = min(x0 + row, height - 1) * width + min(y0 + col, width - 1);
+			const unsigned int image_base = batch * height * width;
+			raw_t residual[4][4];
+			if constexpr (HAS_EXT)
+			{
+#pragma unroll
+				for (int row = 0; row < 4; row++)
+#pragma unroll
+					for (int col = 0; col < 4; col++)
+						residual[row][col] = *reinterpret_cast<const raw_t*>(ext + (image_base + pixel[row][col]) * channels + channel);
+			}
+
+			float tmp[4][6][VEC];
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+			{
+				float line[6][VEC];
+#pragma unroll
+				for (int row = 0; row < 6; row++)
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						line[row][c] = RawVec<T, VEC>::get(raw[row][col], c);
+				float res[4][VEC];
+				output_transform_1d<VEC>(line, res);
+#pragma unroll
+				for (int row = 0; row < 4; row++)
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						tmp[row][col][c] = res[row][c];
+			}
+#pragma unroll
+			for (int row = 0; row < 4; row++)
+			{
+				float res[4][VEC];
+				output_transform_1d<VEC>(tmp[row], res);
+#pragma unroll
+				for (int col = 0; col < 4; col++)
+				{
+					Vec<T, VEC> out;
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+					{
+						float t = res[col][c] + b.v[c];
+						if constexpr (HAS_EXT)
+							t = t + RawVec<T, VEC>::get(residual[row][col], c);
+						if constexpr (ACT == 1)
+							t = fmaxf(t, 0.0f);
+						if constexpr (ACT == 2)
+						{
+							if constexpr (sizeof(T) == 2)
+								t = half_bits_to_float(half_bits_rtz(t));
+							t = activate(act, t);
+						}
+						out.v[c] = t;
+					}
+					if ((x0 + row) < height && (y0 + col) < width)
+					{
+						out.store(image + pixel[row][col] * SLICE + channel_local);
+						if (output != nullptr)
+							out.store(output + (image_base + pixel[row][col]) * channels + channel);
+					}
+				}
+			}
+		}
+		__syncthreads();
+
+		/* ---- phase 2: input transform of the next layer out of LDS ---- */
+#pragma clang loop unroll(disable)
+		for (unsigned int in_image = tile_lane; in_image < tiles_per_image; in_image += TILE_LANES)
+		{
+			const unsigned int tile_idx = batch * tiles_per_image + in_image;
+			const int tile_x = in_image / tiles_w;
+			const int x0 = 4 * tile_x - 1;
+			const int y0 = 4 * (in_image - tile_x * tiles_w) - 1;
+			int row_pixel[6], col_pixel[6];
+			bool row_valid[6], col_valid[6];
+#pragma unroll
+			for (int i = 0; i < 6; i++)
+			{
+				row_valid[i] = (x0 + i >= 0) && (x0 + i < height);
+				col_valid[i] = (y0 + i >= 0) && (y0 + i < width);
+				row_pixel[i] = min(max(x0 + i, 0), height - 1) * width;
+				col_pixel[i] = min(max(y0 + i, 0), width - 1);
+			}
+			raw_t raw[6][6];
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+#pragma unroll
+				for (int col = 0; col < 6; col++)
+				{
+					const int px = (row_valid[row] && col_valid[col]) ? (row_pixel[row] + col_pixel[col]) : zero_pixel;
+					raw[row][col] = *reinterpret_cast<const raw_t*>(image + px * SLICE + channel_local);
+				}
+
+			float tmp[6][6][VEC];
+#pragma unroll
+			for (int col = 0; col < 6; col++)
+			{
+				float line[6][VEC];
+#pragma unroll
+				for (int row = 0; row < 6; row++)
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						line[row][c] = RawVec<T, VEC>::get(raw[row][col], c);
+				float res[6][VEC];
+				input_transform_1d<VEC>(line, res);
+#pragma unroll
+				for (int row = 0; row < 6; row++)
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						tmp[row][col][c] = res[row][c];
+			}
+			T *dst = next_matrices + static_cast<size_t>(tile_idx) * channels + channel;
+#pragma unroll
+			for (int row = 0; row < 6; row++)
+			{
+				float res[6][VEC];
+				input_transform_1d<VEC>(tmp[row], res);
+#pragma unroll
+				for (int col = 0; col < 6; col++)
+				{
+					Vec<T, VEC> out;
+#pragma unroll
+					for (int c = 0; c < VEC; c++)
+						out.v[c] = res[col][c];
+					out.store(dst + static_cast<size_t>(row * 6 + col) * matrix_stride);
+				}
+			}
+		}
+	}
+
 	/* ---------------------------------------------------------------------------------------------------------------------
 	 * host side
 	 * ------------------------------------------------------------------------------------------------------------------- */
@@ -483,6 +678,52 @@ namespace
 		}
 		MLHIP_CHECK(hipGetLastError());
 	}
+	/* fused output + next input transform: channels must be a multiple of 64 and 4-element accesses aligned */
+	template<typename T, int SLICE>
+	void launch_output_input(hipStream_t stream, const mlTensor_t &matrices, const mlTensor_t &bias, const mlTensor_t &ext, const mlShape_t &shape, void *output,
+			mlActivationType_t act, mlTensor_t &next)
+	{
+		constexpr int VEC = 4;
+		const int batch = shape.dim[0], height = shape.dim[1], width = shape.dim[2], channels = shape.dim[3];
+		const int tiles_h = ceil_div(height, 4), tiles_w = ceil_div(width, 4);
+		const size_t lds = static_cast<size_t>(height * width + 1) * SLICE * sizeof(T);
+		MLHIP_REQUIRE(lds <= 160 * 1024, "Winograd fused transform: image too large for LDS");
+		const dim3 grid(static_cast<unsigned int>(batch) * (channels / SLICE)), block(256);
+		const T *in = ptr<const T>(matrices);
+		T *out = reinterpret_cast<T*>(output);
+		const T *b = ptr<const T>(bias);
+		const T *e = ptr<const T>(ext);
+		T *nxt = ptr<T>(next);
+		const int a = static_cast<int>(act);
+		const int mode = (act == ACTIVATION_LINEAR) ? 0 : ((act == ACTIVATION_RELU) ? 1 : 2);
+#define MLHIP_LAUNCH_FUSED(MODE, EXT) \
+		do { \
+			auto kernel = kernel_output_input_transform_4x4_3x3<T, VEC, SLICE, MODE, EXT>; \
+			if (lds > 64 * 1024) \
+				ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(lds)); \
+			hipLaunchKernelGGL(kernel, grid, block, lds, stream, in, out, b, e, a, nxt, batch, height, width, channels, tiles_h, tiles_w); \
+		} while (0)
+		if (e != nullptr)
+		{
+			if (mode == 0)
+				MLHIP_LAUNCH_FUSED(0, true);
+			else if (mode == 1)
+				MLHIP_LAUNCH_FUSED(1, true);
+			else
+				MLHIP_LAUNCH_FUSED(2, true);
+		}
+		else
+		{
+			if (mode == 0)
+				MLHIP_LAUNCH_FUSED(0, false);
+			else if (mode == 1)
+				MLHIP_LAUNCH_FUSED(1, false);
+			else
+				MLHIP_LAUNCH_FUSED(2, false);
+		}
+#undef MLHIP_LAUNCH_FUSED
+		MLHIP_CHECK(hipGetLastError());
+	}
 }
 
 extern "C"
@@ -551,6 +792,55 @@ extern "C"
 			launch_output<half_t>(stream_of(context), matrices, bias, ext, out, act);
 		else
 			launch_output<float>(stream_of(context), matrices, bias, ext, out, act);
+	}
+	void hip_winograd_output_input_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
+			mlShape_t output_shape, void *output, mlActivationType_t act, mlTensor_t next_matrices)
+	{
+		MLHIP_REQUIRE(output_shape.rank == 4, "Winograd fused transform: output shape must be [B, H, W, C]");
+		require_supported(tile_size, matrices, matrices.dtype);
+		require_supported(tile_size, next_matrices, matrices.dtype);
+		MLHIP_REQUIRE(next_matrices.dtype == matrices.dtype, "Winograd fused transform: dtype mismatch");
+		const int channels = output_shape.dim[3];
+		const size_t tiles = static_cast<size_t>(output_shape.dim[0]) * ceil_div(output_shape.dim[1], 4) * ceil_div(output_shape.dim[2], 4);
+		MLHIP_REQUIRE(static_cast<size_t>(matrices.dim[1]) == tiles && matrices.dim[2] == channels && static_cast<size_t>(next_matrices.dim[1]) == tiles
+				&& next_matrices.dim[2] == channels, "Winograd fused transform: both sets of matrices must be [36, B*ceil(H/4)*ceil(W/4), C]");
+		if (bias.data != nullptr)
+			MLHIP_REQUIRE(bias.dtype == matrices.dtype && volume(bias) == static_cast<size_t>(channels), "Winograd fused transform: bias must be [C] of the output dtype");
+		if (ext.data != nullptr)
+			MLHIP_REQUIRE(ext.dtype == matrices.dtype && volume(ext) == volume(output_shape), "Winograd fused transform: ext must have the output's shape and dtype");
+		if (tiles == 0 || channels == 0)
+			return;
+		MLHIP_REQUIRE(volume(output_shape) <= 0xffffffffu && tiles * channels <= 0xffffffffu, "Winograd fused transform: tensor too large for 32-bit element offsets");
+		MLHIP_REQUIRE(matrices.data != nullptr && next_matrices.data != nullptr, "Winograd fused transform: null tensor");
+		const int esize = size_of(matrices.dtype);
+		const bool fusable = (channels % 64 == 0) && pick_vec(channels, matrices.data, next_matrices.data, bias.data, ext.data, esize) == 4
+				&& pick_vec(channels, output, nullptr, nullptr, nullptr, esize) == 4
+				&& static_cast<size_t>(output_shape.dim[1] * output_shape.dim[2] + 1) * 64 * esize <= 160 * 1024;
+		if (!fusable)
+		{ /* shapes the fused kernel does not take: the two stand-alone transforms, which need y in memory */
+			MLHIP_REQUIRE(output != nullptr, "Winograd fused transform: this shape needs the output tensor as intermediate storage");
+			mlTensor_t y = make_tensor(output, matrices.dtype, output_shape);
+			hip_winograd_output_transform(context, tile_size, matrices, bias, ext, y, act);
+			hip_winograd_input_transform(context, tile_size, y, next_matrices);
+			return;
+		}
+		mlTensor_t next = next_matrices;
+		/* wider channel slices make longer contiguous segments in memory, as long as two workgroups still fit the LDS of a CU */
+		const bool wide = false && (channels % 128 == 0) && static_cast<size_t>(output_shape.dim[1] * output_shape.dim[2] + 1) * 128 * esize <= 80 * 1024;
+		if (matrices.dtype == DTYPE_FLOAT16)
+		{
+			if (wide)
+				launch_output_input<half_t, 128>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+			else
+				launch_output_input<half_t, 64>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+		}
+		else
+		{
+			if (wide)
+				launch_output_input<float, 128>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+			else
+				launch_output_input<float, 64>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+		}
 	}
 } /* extern "C" */
 

@@ -44,9 +44,10 @@ def make_input(seed, batch, board, planes, p=0.3):
 
 
 class ResNet:
-    def __init__(self, context, batch, board, input_planes, channels, blocks, dtype, params_host, to_storage, chunk=None):
+    def __init__(self, context, batch, board, input_planes, channels, blocks, dtype, params_host, to_storage, chunk=None, fused=False):
         """params_host: list from make_parameters; to_storage: fp32 ndarray -> ndarray in the storage type (identity or fp16 bits)."""
         self.context = context
+        self.fused = fused
         self.dtype = ml.dtype_of(dtype)
         self.batch, self.board, self.channels, self.blocks = batch, board, channels, blocks
         self.chunk = min(chunk or batch, batch)
@@ -76,8 +77,11 @@ class ResNet:
         per = tensor.volume() // tensor.shape[0]
         return tensor.view((count,) + tensor.shape[1:], start * per)
 
-    def forward(self):
-        """One pass over the whole batch; asynchronous on the context's stream."""
+    def forward(self, fused=None):
+        """One pass over the whole batch; asynchronous on the context's stream. With `fused` (default: the constructor's choice) the
+        output transform of every 3x3 layer is merged with the input transform of the next one; results are bit-identical."""
+        if self.fused if fused is None else fused:
+            return self._forward_fused()
         for start in range(0, self.batch, self.chunk):
             n = min(self.chunk, self.batch - start)
             x = self._view_batch(self.input, start, n)
@@ -92,6 +96,41 @@ class ResNet:
                 a, c = c, a
             ml.set_timer_label("head")
             self.layers[-1].forward([a], self._view_batch(self.output, start, n), self.workspace)
+            ml.set_timer_label(None)
+        return self.output
+
+    def _forward_fused(self):
+        """Same network with cross-layer fusion inside each residual block: the result of the block's first convolution goes from its
+        output transform to the second convolution's input transform through LDS and is never written to memory."""
+        L = self.layers
+        for start in range(0, self.batch, self.chunk):
+            n = min(self.chunk, self.batch - start)
+            x = self._view_batch(self.input, start, n)
+            a, b, c = (self._view_batch(t, 0, n) for t in self.act)
+            ws = self.workspace
+            ml.set_timer_label("stem")
+            # the stem has fewer input than output channels: its output matrices start below the end of the next layer's input
+            # matrices in the shared workspace, so its two transforms stay separate calls
+            L[0].forward([x], a, ws)
+            if self.blocks > 0:
+                ml.set_timer_label("block_conv1")
+                L[1].winograd_input(a, ws)
+            for blk in range(self.blocks):
+                conv1, conv2 = L[1 + 2 * blk], L[2 + 2 * blk]
+                ml.set_timer_label("block_conv1")
+                conv1.winograd_gemm(n, ws)
+                conv1.winograd_output_into(conv2, n, None if self.channels % 64 == 0 else b, None, ws)  # only conv2 reads this result
+                ml.set_timer_label("block_conv2")
+                conv2.winograd_gemm(n, ws)
+                # with a residual to read and the block output to write the fused launch is not faster than the two transforms
+                # (measured: its register footprint halves the occupancy), so the block boundary stays unfused
+                conv2.winograd_output(c, a, ws)  # c = next block's input and residual
+                if blk + 1 < self.blocks:
+                    ml.set_timer_label("block_conv1")
+                    L[3 + 2 * blk].winograd_input(c, ws)
+                a, c = c, a
+            ml.set_timer_label("head")
+            L[-1].forward([a], self._view_batch(self.output, start, n), ws)
             ml.set_timer_label(None)
         return self.output
 

@@ -88,6 +88,23 @@ def test_chunked_execution_is_bit_identical(ctx):
     assert mismatches(outs[0], outs[2]) == 0
 
 
+@pytest.mark.parametrize("dtype,channels,blocks", [("float16", 64, 3), ("float32", 128, 2), ("float16", 40, 2)])
+def test_cross_layer_fusion_is_bit_identical(ctx, dtype, channels, blocks):
+    """Merging each output transform with the next layer's input transform (activations stay in LDS between them) must not change a
+    single bit of the head output or of the last block's output; 40 channels exercise the entry point's two-kernel route."""
+    conv = O.to_half if dtype == "float16" else (lambda a: np.ascontiguousarray(a, np.float32))
+    params = make_parameters(9, 32, channels, blocks)
+    x = conv(make_input(9, 6, 15, 32))
+    net = ResNet(ctx, 6, 15, 32, channels, blocks, dtype, params, conv)
+    net.setInput(x)
+    plain = net.forward(fused=False).copyToHost(ctx)
+    trunk_plain = net.trunk_output().copyToHost(ctx)
+    fused = net.forward(fused=True).copyToHost(ctx)
+    trunk_fused = net.trunk_output().copyToHost(ctx)
+    assert mismatches(plain, fused) == 0
+    assert mismatches(trunk_plain, trunk_fused) == 0
+
+
 def test_full_size_batch_1024_properties(ctx):
     """The benchmark workload itself (config 2: B = 1024): repeated passes are bit-identical (no races, no stale workspace), and the
     first positions reproduce a batch-4 run of the same network bit for bit, which in turn is checked against the oracle."""
@@ -98,6 +115,7 @@ def test_full_size_batch_1024_properties(ctx):
     a = net.forward().copyToHost(ctx)
     b = net.forward().copyToHost(ctx)
     assert mismatches(a, b) == 0
+    assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0  # the benchmark's fused pass computes the same bits
     small = ResNet(ctx, 4, 15, 32, 256, 20, "float16", params, O.to_half)
     small.setInput(x[:4])
     c = small.forward().copyToHost(ctx)

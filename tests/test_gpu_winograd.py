@@ -157,3 +157,41 @@ def test_empty_and_full_size_properties(ctx):
     dx.zeroall(ctx)
     ml.winogradInputTransform(ctx, (256, 3, 3, 256), dx, full)
     assert not full.copyToHost(ctx).any()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("shape", [(2, 15, 15, 64), (3, 19, 19, 128), (2, 9, 11, 64), (1, 4, 4, 64), (2, 7, 5, 192), (2, 9, 11, 35)])
+def test_fused_output_input_transform_bit_exact(ctx, dtype, shape):
+    """hip_winograd_output_input_transform against the oracle's output transform followed by its input transform, bit for bit: with
+    and without bias / residual, ReLU / linear / a transcendental activation (exact against the GPU's own two-call sequence), with
+    y written to memory and with y kept on chip. The last shape (35 channels) takes the entry point's two-kernel route."""
+    rng = np.random.default_rng(sum(shape))
+    b, h, w, c = shape
+    tiles = b * ((h + 3) // 4) * ((w + 3) // 4)
+    m = random_tensor(rng, (36, tiles, c), dtype)
+    bias = random_tensor(rng, (c,), dtype)
+    ext = random_tensor(rng, shape, dtype)
+    dm, db, de = ml.toDevice(ctx, m), ml.toDevice(ctx, bias), ml.toDevice(ctx, ext)
+    wshape = (c, 3, 3, c)
+    for use_bias, use_ext, act in ((True, True, O.RELU), (False, False, O.LINEAR), (True, False, O.RELU), (False, True, O.LINEAR)):
+        want_y = O.winograd_output_transform(m, shape, bias if use_bias else None, ext if use_ext else None, act)
+        want_v = O.winograd_input_transform(want_y)
+        for keep_y in (True, False):
+            if not keep_y and c % 64 != 0:
+                continue
+            dy = ml.Tensor(shape, dtype)
+            dy.setall(ctx, 7.0)
+            dv = ml.Tensor((36, tiles, c), dtype)
+            dv.setall(ctx, float("nan"))
+            ml.winogradOutputInputTransform(ctx, wshape, dm, shape, dy if keep_y else None, db if use_bias else None, de if use_ext else None, act, dv)
+            assert mismatches(dv.copyToHost(ctx), want_v) == 0
+            if keep_y:
+                assert mismatches(dy.copyToHost(ctx), want_y) == 0
+    # activations that the reference runs as a second pass: identical to the GPU's own two calls
+    dy2, dv2 = ml.Tensor(shape, dtype), ml.Tensor((36, tiles, c), dtype)
+    ml.winogradOutputTransform(ctx, wshape, dm, dy2, db, de, O.TANH)
+    ml.winogradInputTransform(ctx, wshape, dy2, dv2)
+    dy3, dv3 = ml.Tensor(shape, dtype), ml.Tensor((36, tiles, c), dtype)
+    ml.winogradOutputInputTransform(ctx, wshape, dm, shape, dy3, db, de, O.TANH, dv3)
+    assert mismatches(dv3.copyToHost(ctx), dv2.copyToHost(ctx)) == 0
+    assert mismatches(dy3.copyToHost(ctx), dy2.copyToHost(ctx)) == 0
