@@ -82,21 +82,18 @@ namespace
 		return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 	}
 
-	template<typename T>
-	void launch_stream_gemm(hipStream_t stream, const GemmArgs &g)
+	/* persistent streaming kernel for 512-byte K rows: 8 wavefronts x 32 columns cover N up to 256 per workgroup, 4 cover N <= 128 */
+	template<typename T, int WAVES>
+	void launch_stream_gemm_as(hipStream_t stream, const GemmArgs &g)
 	{
 		typedef StreamGemmConfig Cfg;
-		constexpr int STAGES = (sizeof(T) == 2) ? 8 : 7; /* the fp32 slabs are twice as large */
-		constexpr int LDS = Cfg::lds_bytes<T>(STAGES);
+		constexpr int SLAB_BYTES = WAVES * 32 * (32 * sizeof(T) + 16);
+		constexpr int STAGES = (8 * Cfg::STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? 8 : 7;
+		constexpr int LDS = STAGES * Cfg::STAGE_BYTES + SLAB_BYTES;
 		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
-		auto kernel = kernel_gemm_stream_nt<T, STAGES>;
-		static bool configured = false; /* per instantiation; the attribute belongs to the function, setting it twice is harmless */
-		if (!configured)
-		{
-			MLHIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS));
-			configured = true;
-		}
-		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, Cfg::BN);
+		auto kernel = kernel_gemm_stream_wide_nt<T, WAVES, STAGES>;
+		ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), LDS);
+		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, 32 * WAVES);
 		const int total_units = g.batch * tiles_m;
 		const int compute_units = device_compute_units();
 		int groups = compute_units / n_tiles;
@@ -107,8 +104,16 @@ namespace
 		if (groups > total_units)
 			groups = total_units;
 		const int units_per_group = ceil_div(total_units, groups);
-		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(Cfg::THREADS), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
+		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
 				reinterpret_cast<T*>(g.D), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group);
+	}
+	template<typename T>
+	void launch_stream_gemm(hipStream_t stream, const GemmArgs &g)
+	{
+		if (g.N <= 128)
+			launch_stream_gemm_as<T, 4>(stream, g);
+		else
+			launch_stream_gemm_as<T, 8>(stream, g);
 	}
 }
 

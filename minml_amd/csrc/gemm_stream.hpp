@@ -62,6 +62,10 @@ namespace mlhip
 				break;
 		}
 	}
+	__device__ __forceinline__ void wait_lgkmcnt_zero()
+	{
+		__builtin_amdgcn_s_waitcnt(0xc07f);
+	}
 	/* s_barrier without a memory fence: the waits above already order the direct-to-LDS loads this kernel cares about */
 	__device__ __forceinline__ void barrier_no_fence()
 	{
@@ -298,6 +302,246 @@ namespace mlhip
 				step(std::integral_constant<int, 1>(), u);
 				step(std::integral_constant<int, 2>(), u);
 				step(std::integral_constant<int, 3>(), u);
+			}
+			unit = run_end;
+		}
+	}
+	/* at most `stages` stages of LOADS vector-memory operations each may remain outstanding */
+	template<int LOADS>
+	__device__ __forceinline__ void wait_vmcnt_stages(int stages)
+	{
+		switch (stages)
+		{
+			case 0:
+				wait_vmcnt<0>();
+				break;
+			case 1:
+				wait_vmcnt<LOADS>();
+				break;
+			case 2:
+				wait_vmcnt<2 * LOADS>();
+				break;
+			case 3:
+				wait_vmcnt<3 * LOADS>();
+				break;
+			case 4:
+				wait_vmcnt<4 * LOADS>();
+				break;
+			case 5:
+				wait_vmcnt<5 * LOADS>();
+				break;
+			case 6:
+				wait_vmcnt<6 * LOADS>();
+				break;
+			default:
+				wait_vmcnt<7 * LOADS>();
+				break;
+		}
+	}
+	template<int N, typename F>
+	__device__ __forceinline__ void stream_static_for(F &&f)
+	{
+		if constexpr (N > 0)
+		{
+			stream_static_for<N - 1>(f);
+			f(std::integral_constant<int, N - 1>());
+		}
+	}
+
+	/*
+	 * Second form of the streaming product: one workgroup of WAVES wavefronts (two per SIMD when WAVES = 8) covers 128 rows x 32 * WAVES
+	 * columns, i.e. all of N = 256 with 8 wavefronts, so every row of A is fetched by exactly one workgroup (half the L2 -> LDS traffic of
+	 * the two-slice form) and a wavefront that waits - on a full memory pipeline, at the stage barrier, in its store epilogue - shares its
+	 * SIMD with one that does not. Each wavefront keeps the B operand of its 32 columns in 64 VGPRs and accumulates 128 x 32 outputs;
+	 * the pipeline is one k step deep (fragments of k step t + 1 are read while k step t is multiplied). Same ring, swizzle and hand-kept
+	 * counters as kernel_gemm_stream_nt.
+	 */
+	template<typename T, int WAVES, int STAGES>
+	__global__ __launch_bounds__(64 * WAVES, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a, size_t stride_b,
+			size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group)
+	{
+		typedef StreamGemmConfig Cfg;
+		typedef MfmaTraits<T> Traits;
+		typedef typename Traits::acc_vec acc_vec;
+		constexpr int BN = 32 * WAVES;
+		constexpr int DISTANCE = STAGES - 1; /* stages requested ahead of the one being multiplied */
+		constexpr int LOADS = 16 / WAVES; /* 1 KB blocks of a 16 KB stage moved by one wavefront */
+		constexpr int SLAB_STRIDE = 32 * sizeof(T) + 16;
+		constexpr int KSTEPS = 4; /* MFMA k steps per stage */
+		static_assert(16 % WAVES == 0 && DISTANCE >= 2 && DISTANCE <= 8 && (DISTANCE - 2) * LOADS <= 63, "unsupported workgroup shape");
+		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+		uint8_t *ring = lds;
+		uint8_t *slab = lds + STAGES * Cfg::STAGE_BYTES + (threadIdx.x >> 6) * (32 * SLAB_STRIDE);
+
+		const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+		int group, n_tile;
+		if (gridDim.x % (8 * n_tiles) == 0)
+		{
+			const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+			group = (slot / n_tiles) * 8 + xcd;
+			n_tile = slot % n_tiles;
+		}
+		else
+		{
+			group = blockIdx.x / n_tiles;
+			n_tile = blockIdx.x % n_tiles;
+		}
+		const int n0 = n_tile * BN + wave * 32; /* first column of this wavefront */
+		const int total_units = batch * tiles_m;
+		const int unit_begin = group * units_per_group;
+		const int unit_end = min(total_units, unit_begin + units_per_group);
+		if (unit_begin >= unit_end)
+			return;
+
+		int load_row[LOADS], load_chunk_bytes[LOADS];
+#pragma unroll
+		for (int i = 0; i < LOADS; i++)
+		{
+			const int row = (wave + WAVES * i) * 8 + (lane >> 3);
+			load_row[i] = row;
+			load_chunk_bytes[i] = ((lane & 7) ^ ((row >> 1) & 7)) * 16;
+		}
+		const int frag_row = lane & 31;
+		const int half_sel = lane >> 5;
+		int frag_first[4]; /* byte offset within a stage of this lane's fragment of k step 0, per 32-row block */
+#pragma unroll
+		for (int i = 0; i < 4; i++)
+		{
+			const int row = 32 * i + frag_row;
+			frag_first[i] = row * Cfg::STAGE_K_BYTES + ((half_sel ^ ((row >> 1) & 7)) * 16);
+		}
+
+		int unit = unit_begin;
+		while (unit < unit_end)
+		{
+			const int matrix = unit / tiles_m;
+			const int run_end = min(unit_end, (matrix + 1) * tiles_m);
+			const int run_units = run_end - unit;
+			const int run_stages = run_units * Cfg::STAGES_PER_UNIT;
+			const int first_tile = unit - matrix * tiles_m;
+			const uint8_t *a_base = reinterpret_cast<const uint8_t*>(A + static_cast<size_t>(matrix) * stride_a);
+			const uint8_t *b_base = reinterpret_cast<const uint8_t*>(B + static_cast<size_t>(matrix) * stride_b);
+			T *c_base = C + static_cast<size_t>(matrix) * stride_c;
+
+			wait_vmcnt<0>();
+			wait_lgkmcnt_zero();
+			barrier_no_fence(); /* nobody reads stages of the previous run any more */
+
+			uint4_t b_regs[16]; /* 32 columns x 16 k steps, 16 bytes per lane each */
+			{
+				const int n = min(n0 + frag_row, N - 1);
+				const uint8_t *row = b_base + static_cast<size_t>(n) * Cfg::K_BYTES + half_sel * 16;
+#pragma unroll
+				for (int k = 0; k < 16; k++)
+					b_regs[k] = *reinterpret_cast<const uint4_t*>(row + k * 32);
+			}
+			auto request_stage = [&](int g)
+			{
+				const int u = g / Cfg::STAGES_PER_UNIT, ks = g - u * Cfg::STAGES_PER_UNIT;
+				const int m_first = (first_tile + u) * Cfg::BM;
+				uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
+#pragma unroll
+				for (int i = 0; i < LOADS; i++)
+				{
+					const int m = min(m_first + load_row[i], M - 1);
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * Cfg::K_BYTES + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
+							(lds_ptr_t) (stage + (wave + WAVES * i) * 1024), 16, 0, 0);
+				}
+			};
+			uint4_t frags[2][4];
+			auto read_fragments = [&](int g, int kk, uint4_t (&regs)[4])
+			{
+				const uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+					regs[i] = *reinterpret_cast<const uint4_t*>(stage + (frag_first[i] ^ (kk * 32)));
+			};
+			acc_vec acc[4];
+			auto clear_accumulators = [&]()
+			{
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						acc[i][r] = 0;
+			};
+			auto store_unit = [&](int u)
+			{
+				/* lane l, register r of block i: m = 32 i + l % 32, n = 8 (r / 4) + 4 (l / 32) + r % 4 */
+				constexpr int ELEMS_PER_16B = 16 / sizeof(T);
+				constexpr int LANES_PER_ROW = 32 / ELEMS_PER_16B;
+				constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+				const int m_first = (first_tile + u) * Cfg::BM;
+				const int col = (lane % LANES_PER_ROW) * ELEMS_PER_16B;
+#pragma unroll
+				for (int i = 0; i < 4; i++)
+				{
+#pragma unroll
+					for (int q = 0; q < 4; q++)
+					{
+						Vec<T, 4> v;
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							v.v[e] = acc[i][4 * q + e];
+						v.store(reinterpret_cast<T*>(slab + frag_row * SLAB_STRIDE) + 8 * q + 4 * half_sel);
+					}
+					wait_lgkmcnt_zero(); /* the slab is private to this wavefront */
+					__builtin_amdgcn_wave_barrier();
+#pragma unroll
+					for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++)
+					{
+						const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW;
+						const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
+						const int m = m_first + 32 * i + row;
+						if (m < M && n0 + col < N) /* N is a multiple of the 16-byte vector (checked by the launcher) */
+							*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n0 + col) = v;
+					}
+					wait_lgkmcnt_zero();
+					__builtin_amdgcn_wave_barrier();
+				}
+			};
+
+			for (int g = 0; g < DISTANCE; g++)
+				if (g < run_stages)
+					request_stage(g);
+			wait_vmcnt<0>(); /* B operand and the first stages: one memory latency per run, and no register loads left for the compiler to guard */
+			barrier_no_fence();
+			clear_accumulators();
+			read_fragments(0, 0, frags[0]);
+
+			for (int u = 0; u < run_units; u++)
+			{
+				stream_static_for<Cfg::STAGES_PER_UNIT * KSTEPS>([&](auto step)
+				{
+					constexpr int t = decltype(step)::value; /* k step within the unit */
+					constexpr int ks = t / KSTEPS, kk = t % KSTEPS;
+					constexpr int cur = t & 1, nxt = 1 - cur;
+					const int g = u * Cfg::STAGES_PER_UNIT + ks;
+					/* the first MFMA is guarded by the compiler with lgkmcnt(0): this k step's fragments were requested one k step ago */
+					Traits::mma(b_regs[t], frags[cur][0], acc[0]);
+					__builtin_amdgcn_sched_barrier(0);
+					if constexpr (kk + 1 < KSTEPS)
+						read_fragments(g, kk + 1, frags[nxt]);
+					else if (g + 1 < run_stages)
+					{
+						/* stage g + 1 has landed once at most the loads of the stages requested after it (g + 2 .. g + DISTANCE - 1) are
+						 * outstanding; after the barrier every wavefront has all of stage g in registers, so the buffers of stages <= g
+						 * are free and stage g + DISTANCE takes that of stage g + DISTANCE - STAGES */
+						wait_lgkmcnt_zero();
+						wait_vmcnt_stages<LOADS>(min(DISTANCE - 2, run_stages - 2 - g));
+						barrier_no_fence();
+						if (g + DISTANCE < run_stages)
+							request_stage(g + DISTANCE);
+						read_fragments(g + 1, 0, frags[nxt]);
+					}
+					__builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+					for (int i = 1; i < 4; i++)
+						Traits::mma(b_regs[t], frags[cur][i], acc[i]);
+					__builtin_amdgcn_sched_barrier(0);
+				});
+				store_unit(u);
+				clear_accumulators();
 			}
 			unit = run_end;
 		}
