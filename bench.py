@@ -172,7 +172,7 @@ def main():
         if n_t:
             transforms["%s@%s" % (entry, label)] = {"kernel": kernel, "launches_timed": n_t, "avg_launch_us": t_t * 1e6, "algorithmic_bytes": nbytes,
                                                    "gbs": nbytes / t_t / 1e9, "frac_hbm": nbytes / t_t / 1e9 / PEAK_HBM_GBS}
-    kernel_name = "kernel_gemm_stream_nt" if channels * esize == 512 else "kernel_gemm_nt"
+    kernel_name = "kernel_gemm_stream_wide_nt" if channels * esize == 512 else "kernel_gemm_nt"
     result = {
         "metric": "positions/sec at batch 1024 (20x256 res-net fp16); % MFMA peak in conv GEMMs" if args.config.startswith("cfg2")
         else "positions/sec (%s)" % args.config,

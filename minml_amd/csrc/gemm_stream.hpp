@@ -4,17 +4,19 @@
  *
  * This product is bound by HBM, not by the matrix cores: one matrix pair moves T*512 bytes in and T*N*s bytes out for only
  * 2*T*N*K flops, and the 36 B operands together are a few megabytes. The kernel is therefore organised around the A stream:
- *   - persistent workgroups (one per CU), each owning a contiguous range of "units" (128 rows of A of one matrix) and one 128-column
- *     slice of N; workgroups that need the same A rows for different column slices sit on one XCD so the second read is an L2 hit;
- *   - every wavefront keeps ITS part of the B operand (64 columns x full K = 128 VGPRs) in registers for the whole run of units that
+ *   - persistent workgroups (one per CU), each owning a contiguous range of "units" (128 rows of A of one matrix) and, with 8
+ *     wavefronts of 32 columns each, all 256 columns of N, so that every row of A is fetched by exactly one workgroup (for wider N the
+ *     column slices of one row range sit on one XCD and share its L2);
+ *   - every wavefront keeps ITS part of the B operand (32 columns x full K = 64 VGPRs) in registers for the whole run of units that
  *     share a matrix, so B costs neither LDS space nor LDS bandwidth;
  *   - A moves HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4, no staging registers) into a ring of 128-byte-per-row
- *     stages that runs ahead across unit boundaries (prefetch distance STAGES - 2 stages of 16 KB), so loads never stop for an
- *     epilogue or for the next tile's prologue; completion is tracked with explicit vmcnt waits and fence-free barriers (a fence
- *     would drain the whole ring);
- *   - fragment reads of stage g are in flight while the MFMAs of stage g - 1 run (register double buffer);
- *   - LDS stages are written linearly by the DMA and read conflict-free through an XOR swizzle of the 16-byte chunk index;
- *   - accumulators leave through a per-wavefront LDS slab so that global stores are 16 bytes per lane and 128-byte contiguous.
+ *     stages that runs ahead across unit boundaries (STAGES - 1 stages of 16 KB), so loads never stop for an epilogue or for the next
+ *     unit's prologue; completion is tracked with explicit vmcnt waits and fence-free barriers (a fence would drain the whole ring);
+ *   - two wavefronts per SIMD: one that waits (full memory pipeline, stage barrier, store epilogue) leaves the SIMD to the other;
+ *   - fragment reads of k step t + 1 are in flight while k step t is multiplied (register double buffer);
+ *   - LDS stages are written linearly by the DMA and read through an XOR swizzle of the 16-byte chunk index (row / 2: measured to be
+ *     the placement that sustains full LDS read bandwidth for the MFMA fragment access on gfx950);
+ *   - accumulators leave through a per-wavefront LDS slab so that global stores are 16 bytes per lane, 64 bytes contiguous per row.
  */
 #ifndef MINML_AMD_GEMM_STREAM_HPP_
 #define MINML_AMD_GEMM_STREAM_HPP_
@@ -33,34 +35,6 @@ namespace mlhip
 	{
 		/* s_waitcnt immediate: vmcnt in bits [3:0] and [15:14], expcnt [6:4] and lgkmcnt [11:8] left at "no wait" */
 		__builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-	}
-	/* at most `loads` vector-memory operations may remain outstanding (a multiple of 4 between 0 and 24) */
-	__device__ __forceinline__ void wait_vmcnt_dynamic(int loads)
-	{
-		switch (loads >> 2)
-		{
-			case 0:
-				wait_vmcnt<0>();
-				break;
-			case 1:
-				wait_vmcnt<4>();
-				break;
-			case 2:
-				wait_vmcnt<8>();
-				break;
-			case 3:
-				wait_vmcnt<12>();
-				break;
-			case 4:
-				wait_vmcnt<16>();
-				break;
-			case 5:
-				wait_vmcnt<20>();
-				break;
-			default:
-				wait_vmcnt<24>();
-				break;
-		}
 	}
 	__device__ __forceinline__ void wait_lgkmcnt_zero()
 	{
@@ -82,230 +56,8 @@ namespace mlhip
 			static constexpr int STAGE_K_BYTES = 128; /* bytes of K per row per stage */
 			static constexpr int STAGE_BYTES = BM * STAGE_K_BYTES; /* 16 KB */
 			static constexpr int STAGES_PER_UNIT = K_BYTES / STAGE_K_BYTES; /* 4 */
-			static constexpr int LOADS_PER_STAGE = 4; /* direct-to-LDS instructions per thread per stage */
-			static constexpr int THREADS = 256;
-			template<typename T>
-			static constexpr int slab_stride()
-			{
-				return 64 * sizeof(T) + 16;
-			}
-			template<typename T>
-			static constexpr int lds_bytes(int stages)
-			{
-				return stages * STAGE_BYTES + 4 * 32 * slab_stride<T>();
-			}
 	};
 
-	template<typename T, int STAGES>
-	__global__ __launch_bounds__(256, 1) void kernel_gemm_stream_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a, size_t stride_b,
-			size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group)
-	{
-		typedef StreamGemmConfig Cfg;
-		typedef MfmaTraits<T> Traits;
-		typedef typename Traits::acc_vec acc_vec;
-		constexpr int DISTANCE = STAGES - 2; /* stages requested ahead of the one being multiplied */
-		constexpr int ELEMS_PER_16B = 16 / sizeof(T);
-		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-		uint8_t *ring = lds;
-		uint8_t *slabs = lds + STAGES * Cfg::STAGE_BYTES;
-
-		const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-		const int wave_m = wave >> 1, wave_n = wave & 1;
-		int group, n_tile;
-		if (gridDim.x % (8 * n_tiles) == 0)
-		{ /* ids congruent mod 8 share an XCD: give the column slices of one group consecutive slots of one XCD */
-			const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-			group = (slot / n_tiles) * 8 + xcd;
-			n_tile = slot % n_tiles;
-		}
-		else
-		{
-			group = blockIdx.x / n_tiles;
-			n_tile = blockIdx.x % n_tiles;
-		}
-		const int n0 = n_tile * Cfg::BN;
-		const int total_units = batch * tiles_m;
-		const int unit_begin = group * units_per_group;
-		const int unit_end = min(total_units, unit_begin + units_per_group);
-		if (unit_begin >= unit_end)
-			return;
-
-		/* loader geometry: per stage the wavefront moves four 1 KB blocks (8 rows x 128 bytes); lane l fills slot l of the block and
-		 * fetches the chunk that the swizzle assigns to that slot */
-		int load_row[Cfg::LOADS_PER_STAGE], load_chunk_bytes[Cfg::LOADS_PER_STAGE];
-#pragma unroll
-		for (int i = 0; i < Cfg::LOADS_PER_STAGE; i++)
-		{
-			const int row = (wave + 4 * i) * 8 + (lane >> 3);
-			load_row[i] = row;
-			load_chunk_bytes[i] = ((lane & 7) ^ ((row >> 1) & 7)) * 16;
-		}
-		/* fragment geometry: lane l supplies row l % 32 and the 16-byte half l / 32 of each 32-byte k step */
-		const int frag_row = lane & 31;
-		const int half_sel = lane >> 5;
-		int frag_offset[2], frag_swizzle[2];
-#pragma unroll
-		for (int i = 0; i < 2; i++)
-		{
-			const int row = wave_m * 64 + i * 32 + frag_row;
-			frag_offset[i] = row * Cfg::STAGE_K_BYTES;
-			frag_swizzle[i] = (row >> 1) & 7;
-		}
-
-		int unit = unit_begin;
-		while (unit < unit_end)
-		{
-			/* ---- a run of units of one matrix ---- */
-			const int matrix = unit / tiles_m;
-			const int run_end = min(unit_end, (matrix + 1) * tiles_m);
-			const int run_units = run_end - unit;
-			const int run_stages = run_units * Cfg::STAGES_PER_UNIT;
-			const int first_tile = unit - matrix * tiles_m;
-			const uint8_t *a_base = reinterpret_cast<const uint8_t*>(A + static_cast<size_t>(matrix) * stride_a);
-			const uint8_t *b_base = reinterpret_cast<const uint8_t*>(B + static_cast<size_t>(matrix) * stride_b);
-			T *c_base = C + static_cast<size_t>(matrix) * stride_c;
-
-			wait_vmcnt<0>();
-			barrier_no_fence(); /* nobody reads stages of the previous run any more */
-
-			/* this wavefront's B operand: 2 blocks of 32 columns x 16 k steps, 16 bytes per lane each */
-			uint4_t b_regs[2][16];
-#pragma unroll
-			for (int j = 0; j < 2; j++)
-			{
-				const int n = min(n0 + wave_n * 64 + j * 32 + frag_row, N - 1);
-				const uint8_t *row = b_base + static_cast<size_t>(n) * Cfg::K_BYTES + half_sel * 16;
-#pragma unroll
-				for (int k = 0; k < 16; k++)
-					b_regs[j][k] = *reinterpret_cast<const uint4_t*>(row + k * 32);
-			}
-
-			auto request_stage = [&](int g)
-			{
-				const int u = g / Cfg::STAGES_PER_UNIT, ks = g - u * Cfg::STAGES_PER_UNIT;
-				const int m_first = (first_tile + u) * Cfg::BM;
-				uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
-#pragma unroll
-				for (int i = 0; i < Cfg::LOADS_PER_STAGE; i++)
-				{
-					const int m = min(m_first + load_row[i], M - 1); /* rows past the end re-read the last row; their products are never stored */
-					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * Cfg::K_BYTES + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
-							(lds_ptr_t) (stage + (wave + 4 * i) * 1024), 16, 0, 0);
-				}
-			};
-			auto read_fragments = [&](int g, uint4_t (&frags)[4][2])
-			{
-				const uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
-#pragma unroll
-				for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-					for (int i = 0; i < 2; i++)
-						frags[kk][i] = *reinterpret_cast<const uint4_t*>(stage + frag_offset[i] + (((2 * kk + half_sel) ^ frag_swizzle[i]) * 16));
-			};
-			acc_vec acc[2][2];
-			auto clear_accumulators = [&]()
-			{
-#pragma unroll
-				for (int i = 0; i < 2; i++)
-#pragma unroll
-					for (int j = 0; j < 2; j++)
-#pragma unroll
-						for (int r = 0; r < 16; r++)
-							acc[i][j][r] = 0;
-			};
-			auto store_unit = [&](int u)
-			{
-				/* lane l, register r of block (i, j): m = 32 i + l % 32, n = 32 j + 8 (r / 4) + 4 (l / 32) + r % 4 */
-				constexpr int SLAB_STRIDE = Cfg::slab_stride<T>();
-				uint8_t *slab = slabs + wave * (32 * SLAB_STRIDE);
-				const int m_first = (first_tile + u) * Cfg::BM + wave_m * 64;
-				constexpr int LANES_PER_ROW = 64 / ELEMS_PER_16B;
-				constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-#pragma unroll
-				for (int i = 0; i < 2; i++)
-				{
-#pragma unroll
-					for (int j = 0; j < 2; j++)
-#pragma unroll
-						for (int q = 0; q < 4; q++)
-						{
-							Vec<T, 4> v;
-#pragma unroll
-							for (int e = 0; e < 4; e++)
-								v.v[e] = acc[i][j][4 * q + e];
-							const int n = 32 * j + 8 * q + 4 * half_sel;
-							v.store(reinterpret_cast<T*>(slab + frag_row * SLAB_STRIDE) + n);
-						}
-					__builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0): the slab is private to this wavefront */
-					__builtin_amdgcn_wave_barrier();
-#pragma unroll
-					for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++)
-					{
-						const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW;
-						const int col = (lane % LANES_PER_ROW) * ELEMS_PER_16B;
-						const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
-						const int m = m_first + 32 * i + row;
-						const int n = n0 + wave_n * 64 + col;
-						if (m < M && n < N) /* N is a multiple of the 16-byte vector (checked by the launcher), so a vector is all in or all out */
-							*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n) = v;
-					}
-					__builtin_amdgcn_s_waitcnt(0xc07f);
-					__builtin_amdgcn_wave_barrier();
-				}
-			};
-
-			for (int g = 0; g < DISTANCE; g++)
-				if (g < run_stages)
-					request_stage(g);
-			/* The B operand must have arrived before the first multiply. Waiting for everything here (B and the first stages, whose
-			 * latencies overlap) costs one memory latency per run and leaves the compiler with no outstanding register loads to track:
-			 * otherwise it guards every multiply in the loop below with a full vmcnt(0), which drains the ring at every stage. */
-			wait_vmcnt<0>();
-			clear_accumulators();
-
-			uint4_t frags[2][4][2];
-			/* one pipeline step for stage position KS of unit u; the position is a compile-time constant so that the register arrays
-			 * (B operand, fragment double buffer) are indexed statically */
-			auto step = [&](auto position, int u)
-			{
-				constexpr int ks = decltype(position)::value;
-				constexpr int pks = (ks + Cfg::STAGES_PER_UNIT - 1) % Cfg::STAGES_PER_UNIT;
-				const int g = u * Cfg::STAGES_PER_UNIT + ks;
-				if (g < run_stages)
-				{
-					/* stage g has landed once at most the loads of the stages requested after it are outstanding */
-					wait_vmcnt_dynamic(min(DISTANCE - 1, run_stages - 1 - g) * Cfg::LOADS_PER_STAGE);
-					barrier_no_fence();
-					if (g + DISTANCE < run_stages)
-						request_stage(g + DISTANCE); /* into the buffer of stage g - 2, whose fragments were consumed before this barrier */
-					read_fragments(g, frags[ks & 1]);
-				}
-				if (g >= 1 && g <= run_stages)
-				{ /* multiply stage g - 1 while the reads of stage g are in flight */
-#pragma unroll
-					for (int kk = 0; kk < 4; kk++)
-#pragma unroll
-						for (int i = 0; i < 2; i++)
-#pragma unroll
-							for (int j = 0; j < 2; j++)
-								Traits::mma(b_regs[j][pks * 4 + kk], frags[pks & 1][kk][i], acc[i][j]);
-					if (pks == Cfg::STAGES_PER_UNIT - 1)
-					{
-						store_unit((g - 1) / Cfg::STAGES_PER_UNIT);
-						clear_accumulators();
-					}
-				}
-			};
-			for (int u = 0; u <= run_units; u++)
-			{
-				step(std::integral_constant<int, 0>(), u);
-				step(std::integral_constant<int, 1>(), u);
-				step(std::integral_constant<int, 2>(), u);
-				step(std::integral_constant<int, 3>(), u);
-			}
-			unit = run_end;
-		}
-	}
 	/* at most `stages` stages of LOADS vector-memory operations each may remain outstanding */
 	template<int LOADS>
 	__device__ __forceinline__ void wait_vmcnt_stages(int stages)
@@ -349,12 +101,8 @@ namespace mlhip
 	}
 
 	/*
-	 * Second form of the streaming product: one workgroup of WAVES wavefronts (two per SIMD when WAVES = 8) covers 128 rows x 32 * WAVES
-	 * columns, i.e. all of N = 256 with 8 wavefronts, so every row of A is fetched by exactly one workgroup (half the L2 -> LDS traffic of
-	 * the two-slice form) and a wavefront that waits - on a full memory pipeline, at the stage barrier, in its store epilogue - shares its
-	 * SIMD with one that does not. Each wavefront keeps the B operand of its 32 columns in 64 VGPRs and accumulates 128 x 32 outputs;
-	 * the pipeline is one k step deep (fragments of k step t + 1 are read while k step t is multiplied). Same ring, swizzle and hand-kept
-	 * counters as kernel_gemm_stream_nt.
+	 * One workgroup of WAVES wavefronts (two per SIMD when WAVES = 8) covers 128 rows x 32 * WAVES columns. Each wavefront keeps the B
+	 * operand of its 32 columns in 64 VGPRs and accumulates 128 x 32 outputs; the pipeline is one k step deep.
 	 */
 	template<typename T, int WAVES, int STAGES>
 	__global__ __launch_bounds__(64 * WAVES, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a, size_t stride_b,
