@@ -8,6 +8,8 @@
 
 #include "device_utils.hpp"
 
+#include <type_traits>
+
 namespace mlhip
 {
 	/*
@@ -51,8 +53,12 @@ namespace mlhip
 			};
 			struct Extra
 			{
-					Vec<T, 4> c;
+					typename std::conditional<sizeof(T) == 2, uint2_t, float4_t>::type raw; /* 4 elements of C, unconverted */
 			};
+			__device__ __forceinline__ bool has_extra() const
+			{
+				return beta != 0.0f;
+			}
 			__device__ __forceinline__ Column load_column(int n) const
 			{
 				Column col;
@@ -65,12 +71,11 @@ namespace mlhip
 					col.bias[e] = b.v[e];
 				return col;
 			}
+			/* only when has_extra(): an unconditional load, kept raw so that nothing waits for it before apply() */
 			__device__ __forceinline__ Extra load_extra(int m, int n) const
 			{
 				Extra x;
-				x.c.zero();
-				if (beta != 0.0f)
-					x.c.load(C + static_cast<size_t>(m) * row_stride + n);
+				x.raw = *reinterpret_cast<const decltype(x.raw)*>(C + static_cast<size_t>(m) * row_stride + n);
 				return x;
 			}
 			__device__ __forceinline__ void apply(int m, int n, const float (&acc)[4], const Column &col, const Extra &x) const
@@ -87,9 +92,23 @@ namespace mlhip
 				}
 				if (beta != 0.0f)
 				{
+					float c[4];
+					if constexpr (sizeof(T) == 2)
+					{
+						c[0] = lo_half(x.raw[0]);
+						c[1] = hi_half(x.raw[0]);
+						c[2] = lo_half(x.raw[1]);
+						c[3] = hi_half(x.raw[1]);
+					}
+					else
+					{
+#pragma unroll
+						for (int e = 0; e < 4; e++)
+							c[e] = x.raw[e];
+					}
 #pragma unroll
 					for (int e = 0; e < 4; e++)
-						out.v[e] += beta * x.c.v[e];
+						out.v[e] += beta * c[e];
 				}
 #pragma unroll
 				for (int e = 0; e < 4; e++)
@@ -163,6 +182,10 @@ namespace mlhip
 			__device__ __forceinline__ Column load_column(int) const
 			{
 				return Column { };
+			}
+			__device__ __forceinline__ bool has_extra() const
+			{
+				return false;
 			}
 			__device__ __forceinline__ Extra load_extra(int, int) const
 			{
@@ -265,12 +288,14 @@ namespace mlhip
 				col.bias = *reinterpret_cast<const float4_t*>(bias + n);
 				return col;
 			}
+			__device__ __forceinline__ bool has_extra() const
+			{
+				return ext != nullptr;
+			}
 			__device__ __forceinline__ Extra load_extra(int m, int n) const
 			{
 				Extra x;
-				x.packed = 0;
-				if (ext != nullptr)
-					x.packed = *reinterpret_cast<const uint32_t*>(ext + static_cast<size_t>(m) * row_stride + n);
+				x.packed = *reinterpret_cast<const uint32_t*>(ext + static_cast<size_t>(m) * row_stride + n);
 				return x;
 			}
 			__device__ __forceinline__ void apply(int m, int n, const int (&acc)[4], const Column &col, const Extra &x) const

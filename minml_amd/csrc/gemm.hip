@@ -82,38 +82,20 @@ namespace
 		return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 	}
 
-	/* persistent streaming kernel for 512-byte K rows: 8 wavefronts x 32 columns cover N up to 256 per workgroup, 4 cover N <= 128 */
-	template<typename T, int WAVES>
-	void launch_stream_gemm_as(hipStream_t stream, const GemmArgs &g)
-	{
-		typedef StreamGemmConfig Cfg;
-		constexpr int SLAB_BYTES = WAVES * 32 * (32 * sizeof(T) + 16);
-		constexpr int STAGES = (8 * Cfg::STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? 8 : 7;
-		constexpr int LDS = STAGES * Cfg::STAGE_BYTES + SLAB_BYTES;
-		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
-		auto kernel = kernel_gemm_stream_wide_nt<T, WAVES, STAGES>;
-		ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), LDS);
-		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, 32 * WAVES);
-		const int total_units = g.batch * tiles_m;
-		const int compute_units = device_compute_units();
-		int groups = compute_units / n_tiles;
-		if (groups >= 8)
-			groups -= groups % 8; /* keeps the grid a multiple of 8 * n_tiles so that the column slices of a group share an XCD */
-		if (groups < 1)
-			groups = 1;
-		if (groups > total_units)
-			groups = total_units;
-		const int units_per_group = ceil_div(total_units, groups);
-		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
-				reinterpret_cast<T*>(g.D), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group);
-	}
 	template<typename T>
-	void launch_stream_gemm(hipStream_t stream, const GemmArgs &g)
+	FloatEpilogue<T> make_float_epilogue(const GemmArgs &g, bool vectorized)
 	{
-		if (g.N <= 128)
-			launch_stream_gemm_as<T, 4>(stream, g);
-		else
-			launch_stream_gemm_as<T, 8>(stream, g);
+		FloatEpilogue<T> ep;
+		ep.D = reinterpret_cast<T*>(g.D);
+		ep.C = reinterpret_cast<const T*>(g.C);
+		ep.bias = reinterpret_cast<const T*>(g.bias);
+		ep.N = g.N;
+		ep.row_stride = g.N;
+		ep.alpha = g.alpha;
+		ep.beta = g.beta;
+		ep.act = g.act;
+		ep.vectorized = vectorized;
+		return ep;
 	}
 }
 
@@ -133,23 +115,47 @@ namespace mlhip
 		const bool fast = nt && g.K > 0 && (k_bytes % 16 == 0) && aligned_to(g.A, 16) && aligned_to(g.B, 16)
 				&& ((g.stride_a * esize) % 16 == 0) && ((g.stride_b * esize) % 16 == 0);
 
-		/* The Winograd product (plain store, 512-byte rows of K, enough rows to fill the chip) takes the persistent streaming kernel. */
-		const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR);
-		if (fast && plain && k_bytes == 512 && (g.dtype == DTYPE_FLOAT16 || g.dtype == DTYPE_FLOAT32) && (g.N * esize) % 16 == 0
-				&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0) && (g.stride_a != 0 || g.batch == 1)
-				&& static_cast<size_t>(g.batch) * ceil_div(g.M, 128) >= 256)
-		{
-			if (g.dtype == DTYPE_FLOAT16)
-				launch_stream_gemm<half_t>(stream, g);
-			else
-				launch_stream_gemm<float>(stream, g);
-			MLHIP_CHECK(hipGetLastError());
-			return;
-		}
-
 		const int out_size = (g.dtype == DTYPE_INT8) ? 4 : esize;
 		const bool vectorized = (g.N % 4 == 0) && aligned_to(g.D, 4 * out_size) && aligned_to(g.C, 4 * out_size) && aligned_to(g.bias, 4 * esize)
 				&& ((g.stride_c * out_size) % (4 * out_size) == 0);
+
+		/*
+		 * Products with short K rows (128 / 256 / 512 bytes) and many rows are bound by HBM: they take the persistent streaming kernel -
+		 * the Winograd products with a plain 16-byte store, everything else (gemm_ex, 1x1 convolutions, the int8 product) with the
+		 * fused epilogue on 4 consecutive outputs.
+		 */
+		if (fast && stream_gemm_applies(g.M, g.batch, k_bytes) && (g.stride_a != 0 || g.batch == 1))
+		{
+			const StreamGemmArgs sg { g.A, g.B, g.D, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a, g.stride_b, g.stride_c };
+			const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR) && (g.N * esize) % 16 == 0
+					&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0);
+			bool launched = true;
+			if (g.dtype == DTYPE_FLOAT16 && plain)
+				launch_stream_gemm<half_t>(stream, sg, PlainStore { });
+			else if (g.dtype == DTYPE_FLOAT32 && plain)
+				launch_stream_gemm<float>(stream, sg, PlainStore { });
+			else if (g.dtype == DTYPE_FLOAT16 && vectorized)
+				launch_stream_gemm<half_t>(stream, sg, make_float_epilogue<half_t>(g, true));
+			else if (g.dtype == DTYPE_FLOAT32 && vectorized)
+				launch_stream_gemm<float>(stream, sg, make_float_epilogue<float>(g, true));
+			else if (g.dtype == DTYPE_INT8 && vectorized && g.bias == nullptr && g.act == ACTIVATION_LINEAR)
+			{
+				Int32Epilogue ep;
+				ep.D = reinterpret_cast<int32_t*>(g.D);
+				ep.N = g.N;
+				ep.row_stride = g.N;
+				ep.vectorized = true;
+				launch_stream_gemm<int8_t>(stream, sg, ep);
+			}
+			else
+				launched = false;
+			if (launched)
+			{
+				MLHIP_CHECK(hipGetLastError());
+				return;
+			}
+		}
+
 
 		/* strides of op(A)[m][k] and op(B)^T[n][k] in elements, for the generic kernel */
 		const size_t a_row = g.transpose_a ? 1 : g.K, a_col = g.transpose_a ? g.M : 1;

@@ -292,6 +292,8 @@ namespace mlhip
 			auto request_extras = [&](auto block, auto buffer)
 			{
 				constexpr int i = decltype(block)::value, buf = decltype(buffer)::value;
+				if (!epilogue.has_extra())
+					return;
 #pragma unroll
 				for (int pass = 0; pass < PASSES; pass++)
 					extra[buf][pass] = epilogue.load_extra(min(m_base + 32 * i + pass * ROWS_PER_PASS, M - 1), n_safe);

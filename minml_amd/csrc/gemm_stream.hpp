@@ -21,6 +21,7 @@
 #ifndef MINML_AMD_GEMM_STREAM_HPP_
 #define MINML_AMD_GEMM_STREAM_HPP_
 
+#include "common.hpp"
 #include "gemm_core.hpp"
 
 #include <type_traits>
@@ -100,31 +101,47 @@ namespace mlhip
 		}
 	}
 
+	/* tag: store the product as is (alpha = 1, beta = 0, no bias, linear), 16 bytes per lane */
+	struct PlainStore
+	{
+	};
+
 	/*
-	 * One workgroup of WAVES wavefronts (two per SIMD when WAVES = 8) covers 128 rows x 32 * WAVES columns. Each wavefront keeps the B
-	 * operand of its 32 columns in 64 VGPRs and accumulates 128 x 32 outputs; the pipeline is one k step deep.
+	 * One workgroup of WAVES_M x WAVES_N wavefronts covers a unit of 128 rows x 32 * WAVES_N columns; a wavefront owns 128 / WAVES_M
+	 * rows x 32 columns, keeps the B operand of its 32 columns (KB bytes of K each) in KB / 8 VGPRs and accumulates in 32x32 blocks; the
+	 * pipeline is one k step deep. KB = 128, 256 or 512 bytes per K row. Epilogue: PlainStore, or a functor with the split protocol of
+	 * epilogues.hpp (load_column / load_extra / apply on 4 consecutive n, vectorized case only), whose D / C pointers advance by
+	 * stride_c per matrix of the batch.
 	 */
-	template<typename T, int WAVES, int STAGES>
-	__global__ __launch_bounds__(64 * WAVES, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a, size_t stride_b,
-			size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group)
+	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue>
+	__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a,
+			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, Epilogue epilogue)
 	{
 		typedef StreamGemmConfig Cfg;
 		typedef MfmaTraits<T> Traits;
 		typedef typename Traits::acc_vec acc_vec;
-		constexpr int BN = 32 * WAVES;
+		typedef typename Traits::acc_t acc_t;
+		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
+		constexpr int WAVES = WAVES_M * WAVES_N;
+		constexpr int BN = 32 * WAVES_N;
+		constexpr int ROWS = Cfg::BM / WAVES_M; /* rows of a unit owned by one wavefront */
+		constexpr int BLOCKS = ROWS / 32;
+		constexpr int STAGES_PER_UNIT = KB / Cfg::STAGE_K_BYTES;
 		constexpr int DISTANCE = STAGES - 1; /* stages requested ahead of the one being multiplied */
 		constexpr int LOADS = 16 / WAVES; /* 1 KB blocks of a 16 KB stage moved by one wavefront */
-		constexpr int SLAB_STRIDE = 32 * sizeof(T) + 16;
+		constexpr int SLAB_STRIDE = 32 * (PLAIN ? sizeof(T) : 4) + 16;
 		constexpr int KSTEPS = 4; /* MFMA k steps per stage */
+		static_assert(KB % Cfg::STAGE_K_BYTES == 0 && ROWS % 32 == 0, "unsupported unit shape");
 		static_assert(16 % WAVES == 0 && DISTANCE >= 2 && DISTANCE <= 8 && (DISTANCE - 2) * LOADS <= 63, "unsupported workgroup shape");
 		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 		uint8_t *ring = lds;
 		uint8_t *slab = lds + STAGES * Cfg::STAGE_BYTES + (threadIdx.x >> 6) * (32 * SLAB_STRIDE);
 
 		const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+		const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
 		int group, n_tile;
 		if (gridDim.x % (8 * n_tiles) == 0)
-		{
+		{ /* ids congruent mod 8 share an XCD: give the column slices of one group consecutive slots of one XCD */
 			const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
 			group = (slot / n_tiles) * 8 + xcd;
 			n_tile = slot % n_tiles;
@@ -134,7 +151,7 @@ namespace mlhip
 			group = blockIdx.x / n_tiles;
 			n_tile = blockIdx.x % n_tiles;
 		}
-		const int n0 = n_tile * BN + wave * 32; /* first column of this wavefront */
+		const int n0 = n_tile * BN + wave_n * 32; /* first column of this wavefront */
 		const int total_units = batch * tiles_m;
 		const int unit_begin = group * units_per_group;
 		const int unit_end = min(total_units, unit_begin + units_per_group);
@@ -151,101 +168,187 @@ namespace mlhip
 		}
 		const int frag_row = lane & 31;
 		const int half_sel = lane >> 5;
-		int frag_first[4]; /* byte offset within a stage of this lane's fragment of k step 0, per 32-row block */
+		int frag_first[BLOCKS]; /* byte offset within a stage of this lane's fragment of k step 0, per 32-row block */
 #pragma unroll
-		for (int i = 0; i < 4; i++)
+		for (int i = 0; i < BLOCKS; i++)
 		{
-			const int row = 32 * i + frag_row;
+			const int row = wave_m * ROWS + 32 * i + frag_row;
 			frag_first[i] = row * Cfg::STAGE_K_BYTES + ((half_sel ^ ((row >> 1) & 7)) * 16);
 		}
 
 		int unit = unit_begin;
 		while (unit < unit_end)
 		{
+			/* ---- a run of units of one matrix ---- */
 			const int matrix = unit / tiles_m;
 			const int run_end = min(unit_end, (matrix + 1) * tiles_m);
 			const int run_units = run_end - unit;
-			const int run_stages = run_units * Cfg::STAGES_PER_UNIT;
+			const int run_stages = run_units * STAGES_PER_UNIT;
 			const int first_tile = unit - matrix * tiles_m;
 			const uint8_t *a_base = reinterpret_cast<const uint8_t*>(A + static_cast<size_t>(matrix) * stride_a);
 			const uint8_t *b_base = reinterpret_cast<const uint8_t*>(B + static_cast<size_t>(matrix) * stride_b);
 			T *c_base = C + static_cast<size_t>(matrix) * stride_c;
+			Epilogue local = epilogue;
+			if constexpr (!PLAIN)
+			{
+				local.D += static_cast<size_t>(matrix) * stride_c;
+				if constexpr (Epilogue::has_c)
+					local.C += static_cast<size_t>(matrix) * stride_c;
+			}
 
 			wait_vmcnt<0>();
 			wait_lgkmcnt_zero();
 			barrier_no_fence(); /* nobody reads stages of the previous run any more */
 
-			uint4_t b_regs[16]; /* 32 columns x 16 k steps, 16 bytes per lane each */
+			uint4_t b_regs[KB / 32]; /* 32 columns x KB / 32 k steps, 16 bytes per lane each */
 			{
 				const int n = min(n0 + frag_row, N - 1);
-				const uint8_t *row = b_base + static_cast<size_t>(n) * Cfg::K_BYTES + half_sel * 16;
+				const uint8_t *row = b_base + static_cast<size_t>(n) * KB + half_sel * 16;
 #pragma unroll
-				for (int k = 0; k < 16; k++)
+				for (int k = 0; k < KB / 32; k++)
 					b_regs[k] = *reinterpret_cast<const uint4_t*>(row + k * 32);
 			}
-			auto request_stage = [&](int g)
+			auto request_stage = [&](int g) __attribute__((always_inline))
 			{
-				const int u = g / Cfg::STAGES_PER_UNIT, ks = g - u * Cfg::STAGES_PER_UNIT;
+				const int u = g / STAGES_PER_UNIT, ks = g - u * STAGES_PER_UNIT;
 				const int m_first = (first_tile + u) * Cfg::BM;
 				uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
 #pragma unroll
 				for (int i = 0; i < LOADS; i++)
 				{
-					const int m = min(m_first + load_row[i], M - 1);
-					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * Cfg::K_BYTES + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
+					const int m = min(m_first + load_row[i], M - 1); /* rows past the end re-read the last row; their products are never stored */
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * KB + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
 							(lds_ptr_t) (stage + (wave + WAVES * i) * 1024), 16, 0, 0);
 				}
 			};
-			uint4_t frags[2][4];
-			auto read_fragments = [&](int g, int kk, uint4_t (&regs)[4])
+			uint4_t frags[2][BLOCKS];
+			auto read_fragments = [&](int g, int kk, uint4_t (&regs)[BLOCKS]) __attribute__((always_inline))
 			{
 				const uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
 #pragma unroll
-				for (int i = 0; i < 4; i++)
+				for (int i = 0; i < BLOCKS; i++)
 					regs[i] = *reinterpret_cast<const uint4_t*>(stage + (frag_first[i] ^ (kk * 32)));
 			};
-			acc_vec acc[4];
-			auto clear_accumulators = [&]()
+			acc_vec acc[BLOCKS];
+			auto clear_accumulators = [&]() __attribute__((always_inline))
 			{
 #pragma unroll
-				for (int i = 0; i < 4; i++)
+				for (int i = 0; i < BLOCKS; i++)
 #pragma unroll
 					for (int r = 0; r < 16; r++)
 						acc[i][r] = 0;
 			};
-			auto store_unit = [&](int u)
+			/*
+			 * Side inputs of the epilogue (per-column constants, residual of every pass of the unit). Loads return in order, so a load
+			 * issued at store time would have to wait for the whole ring in front of it; the residual of unit u is therefore requested
+			 * when unit u starts, from clamped addresses, and is old by the time it is used.
+			 */
+			struct NoSide
+			{
+					struct Column
+					{
+					};
+					struct Extra
+					{
+					};
+			};
+			struct Side
+			{
+					typename std::conditional<PLAIN, NoSide, Epilogue>::type::Column column;
+					typename std::conditional<PLAIN, NoSide, Epilogue>::type::Extra extra[BLOCKS][4];
+			};
+			typename std::conditional<PLAIN, NoSide, Side>::type side;
+			const int side_n = (n0 + (lane & 7) * 4 < N) ? n0 + (lane & 7) * 4 : 0;
+			auto request_side_inputs = [&](int u) __attribute__((always_inline))
+			{
+				if constexpr (!PLAIN)
+				{
+					if (!local.has_extra())
+						return;
+					const int m_first = (first_tile + u) * Cfg::BM + wave_m * ROWS;
+#pragma unroll
+					for (int i = 0; i < BLOCKS; i++)
+#pragma unroll
+						for (int pass = 0; pass < 4; pass++)
+							side.extra[i][pass] = local.load_extra(min(m_first + 32 * i + pass * 8 + (lane >> 3), M - 1), side_n);
+				}
+			};
+			if constexpr (!PLAIN)
+				side.column = local.load_column(side_n);
+			auto store_unit = [&](int u) __attribute__((always_inline))
 			{
 				/* lane l, register r of block i: m = 32 i + l % 32, n = 8 (r / 4) + 4 (l / 32) + r % 4 */
-				constexpr int ELEMS_PER_16B = 16 / sizeof(T);
-				constexpr int LANES_PER_ROW = 32 / ELEMS_PER_16B;
-				constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-				const int m_first = (first_tile + u) * Cfg::BM;
-				const int col = (lane % LANES_PER_ROW) * ELEMS_PER_16B;
-#pragma unroll
-				for (int i = 0; i < 4; i++)
+				const int m_first = (first_tile + u) * Cfg::BM + wave_m * ROWS;
+				if constexpr (PLAIN)
 				{
+					constexpr int ELEMS_PER_16B = 16 / sizeof(T);
+					constexpr int LANES_PER_ROW = 32 / ELEMS_PER_16B;
+					constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+					const int col = (lane % LANES_PER_ROW) * ELEMS_PER_16B;
 #pragma unroll
-					for (int q = 0; q < 4; q++)
+					for (int i = 0; i < BLOCKS; i++)
 					{
-						Vec<T, 4> v;
 #pragma unroll
-						for (int e = 0; e < 4; e++)
-							v.v[e] = acc[i][4 * q + e];
-						v.store(reinterpret_cast<T*>(slab + frag_row * SLAB_STRIDE) + 8 * q + 4 * half_sel);
+						for (int q = 0; q < 4; q++)
+						{
+							Vec<T, 4> v;
+#pragma unroll
+							for (int e = 0; e < 4; e++)
+								v.v[e] = acc[i][4 * q + e];
+							v.store(reinterpret_cast<T*>(slab + frag_row * SLAB_STRIDE) + 8 * q + 4 * half_sel);
+						}
+						wait_lgkmcnt_zero(); /* the slab is private to this wavefront */
+						__builtin_amdgcn_wave_barrier();
+#pragma unroll
+						for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++)
+						{
+							const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW;
+							const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
+							const int m = m_first + 32 * i + row;
+							if (m < M && n0 + col < N) /* N is a multiple of the 16-byte vector (checked by the launcher) */
+								*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n0 + col) = v;
+						}
+						wait_lgkmcnt_zero();
+						__builtin_amdgcn_wave_barrier();
 					}
-					wait_lgkmcnt_zero(); /* the slab is private to this wavefront */
-					__builtin_amdgcn_wave_barrier();
+				}
+				else
+				{
+					/* accumulators cross the slab unconverted; every lane then owns 4 consecutive n of one row per pass */
+					typedef acc_t vec4 __attribute__((ext_vector_type(4)));
+					constexpr int ROWS_PER_PASS = 8, PASSES = 4;
+					const int col = (lane & 7) * 4;
+					const int n = n0 + col;
+					const bool n_valid = n < local.N;
 #pragma unroll
-					for (int pass = 0; pass < 32 / ROWS_PER_PASS; pass++)
+					for (int i = 0; i < BLOCKS; i++)
 					{
-						const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW;
-						const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
-						const int m = m_first + 32 * i + row;
-						if (m < M && n0 + col < N) /* N is a multiple of the 16-byte vector (checked by the launcher) */
-							*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n0 + col) = v;
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+						{
+							vec4 v;
+#pragma unroll
+							for (int e = 0; e < 4; e++)
+								v[e] = acc[i][4 * q + e];
+							*reinterpret_cast<vec4*>(slab + frag_row * SLAB_STRIDE + (8 * q + 4 * half_sel) * 4) = v;
+						}
+						wait_lgkmcnt_zero();
+						__builtin_amdgcn_wave_barrier();
+#pragma unroll
+						for (int pass = 0; pass < PASSES; pass++)
+						{
+							const int row = pass * ROWS_PER_PASS + (lane >> 3);
+							const vec4 v = *reinterpret_cast<const vec4*>(slab + row * SLAB_STRIDE + col * 4);
+							const int m = m_first + 32 * i + row;
+							if (m < M && n_valid)
+							{
+								const acc_t vals[4] = { v[0], v[1], v[2], v[3] };
+								local.apply(m, n, vals, side.column, side.extra[i][pass]);
+							}
+						}
+						wait_lgkmcnt_zero();
+						__builtin_amdgcn_wave_barrier();
 					}
-					wait_lgkmcnt_zero();
-					__builtin_amdgcn_wave_barrier();
 				}
 			};
 
@@ -257,41 +360,129 @@ namespace mlhip
 			clear_accumulators();
 			read_fragments(0, 0, frags[0]);
 
-			for (int u = 0; u < run_units; u++)
+			/*
+			 * One unit: its k steps, then its epilogue. In the STEADY form every stage opening and every request is unconditional, so the
+			 * body is straight-line code and the compiler can count the vector-memory operations between the side-input loads and
+			 * their first use exactly (with branches in between it falls back to vmcnt(0), which drains the ring once per unit); the
+			 * general form serves the last units of a run.
+			 */
+			auto process_unit = [&](int u, auto steady_tag) __attribute__((always_inline))
 			{
-				stream_static_for<Cfg::STAGES_PER_UNIT * KSTEPS>([&](auto step)
+				constexpr bool STEADY = decltype(steady_tag)::value;
+				request_side_inputs(u);
+				stream_static_for<STAGES_PER_UNIT * KSTEPS>([&](auto step)
 				{
 					constexpr int t = decltype(step)::value; /* k step within the unit */
 					constexpr int ks = t / KSTEPS, kk = t % KSTEPS;
 					constexpr int cur = t & 1, nxt = 1 - cur;
-					const int g = u * Cfg::STAGES_PER_UNIT + ks;
+					const int g = u * STAGES_PER_UNIT + ks;
 					/* the first MFMA is guarded by the compiler with lgkmcnt(0): this k step's fragments were requested one k step ago */
 					Traits::mma(b_regs[t], frags[cur][0], acc[0]);
 					__builtin_amdgcn_sched_barrier(0);
 					if constexpr (kk + 1 < KSTEPS)
 						read_fragments(g, kk + 1, frags[nxt]);
-					else if (g + 1 < run_stages)
+					else if (STEADY || g + 1 < run_stages)
 					{
 						/* stage g + 1 has landed once at most the loads of the stages requested after it (g + 2 .. g + DISTANCE - 1) are
 						 * outstanding; after the barrier every wavefront has all of stage g in registers, so the buffers of stages <= g
 						 * are free and stage g + DISTANCE takes that of stage g + DISTANCE - STAGES */
 						wait_lgkmcnt_zero();
-						wait_vmcnt_stages<LOADS>(min(DISTANCE - 2, run_stages - 2 - g));
+						if constexpr (STEADY)
+							wait_vmcnt<(DISTANCE - 2) * LOADS>();
+						else
+							wait_vmcnt_stages<LOADS>(min(DISTANCE - 2, run_stages - 2 - g));
 						barrier_no_fence();
-						if (g + DISTANCE < run_stages)
+						if (STEADY || g + DISTANCE < run_stages)
 							request_stage(g + DISTANCE);
 						read_fragments(g + 1, 0, frags[nxt]);
 					}
 					__builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-					for (int i = 1; i < 4; i++)
+					for (int i = 1; i < BLOCKS; i++)
 						Traits::mma(b_regs[t], frags[cur][i], acc[i]);
 					__builtin_amdgcn_sched_barrier(0);
 				});
 				store_unit(u);
 				clear_accumulators();
-			}
+			};
+			/* steady while the last stage of the unit can still request DISTANCE stages ahead */
+			const int steady_units = max(0, (run_stages - DISTANCE) / STAGES_PER_UNIT);
+			int u = 0;
+			for (; u < steady_units; u++)
+				process_unit(u, std::true_type());
+			for (; u < run_units; u++)
+				process_unit(u, std::false_type());
 			unit = run_end;
+		}
+	}
+	/* operands of one streaming launch: `batch` products C[i] = A[i] * B[i]^T with K rows of k_bytes bytes (strides in elements) */
+	struct StreamGemmArgs
+	{
+			const void *A, *B;
+			void *C; /* used by PlainStore only; functors carry their own pointers */
+			int M, N, k_bytes, batch;
+			size_t stride_a, stride_b, stride_c;
+	};
+	/* enough 128-row units to give every CU several, and a K row length the kernel is instantiated for */
+	inline bool stream_gemm_applies(int M, int batch, size_t k_bytes)
+	{
+		return (k_bytes == 128 || k_bytes == 256 || k_bytes == 512) && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256;
+	}
+	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue>
+	inline void launch_stream_gemm_as(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
+	{
+		typedef StreamGemmConfig Cfg;
+		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
+		constexpr int WAVES = WAVES_M * WAVES_N;
+		constexpr int SLAB_BYTES = WAVES * 32 * (32 * (PLAIN ? sizeof(T) : 4) + 16);
+		constexpr int STAGES = (8 * Cfg::STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? 8 : 7;
+		constexpr int LDS = STAGES * Cfg::STAGE_BYTES + SLAB_BYTES;
+		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
+		auto kernel = kernel_gemm_stream_wide_nt<T, KB, WAVES_M, WAVES_N, STAGES, Epilogue>;
+		ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), LDS);
+		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, 32 * WAVES_N);
+		const int total_units = g.batch * tiles_m;
+		int groups = device_compute_units() / n_tiles;
+		if (groups >= 8)
+			groups -= groups % 8; /* keeps the grid a multiple of 8 * n_tiles so that the column slices of a group share an XCD */
+		if (groups < 1)
+			groups = 1;
+		if (groups > total_units)
+			groups = total_units;
+		const int units_per_group = ceil_div(total_units, groups);
+		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
+				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, epilogue);
+	}
+	/* wavefront layout by output width: 8 x 32 columns for N > 128, 2 x 4 for N > 64, 4 x 2 below */
+	template<typename T, int KB, typename Epilogue>
+	inline void launch_stream_gemm_kb(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
+	{
+		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
+		if (g.N > 128 && (PLAIN || KB < 512))
+			launch_stream_gemm_as<T, KB, 1, 8>(stream, g, epilogue);
+		else if (g.N > 128) /* 64 B-operand registers + side inputs + a 128-row accumulator do not fit 256 VGPRs: two column slices */
+			launch_stream_gemm_as<T, KB, 2, 4>(stream, g, epilogue);
+		else if (g.N > 64)
+			launch_stream_gemm_as<T, KB, 2, 4>(stream, g, epilogue);
+		else
+			launch_stream_gemm_as<T, KB, 4, 2>(stream, g, epilogue);
+	}
+	template<typename T, typename Epilogue>
+	inline void launch_stream_gemm(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
+	{
+		switch (g.k_bytes)
+		{
+			case 128:
+				launch_stream_gemm_kb<T, 128>(stream, g, epilogue);
+				break;
+			case 256:
+				launch_stream_gemm_kb<T, 256>(stream, g, epilogue);
+				break;
+			case 512:
+				launch_stream_gemm_kb<T, 512>(stream, g, epilogue);
+				break;
+			default:
+				fail_logic("HIP backend: streaming GEMM: unsupported K row length");
 		}
 	}
 } /* namespace mlhip */

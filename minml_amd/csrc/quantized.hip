@@ -171,7 +171,12 @@ namespace
 		const size_t k_bytes = static_cast<size_t>(filters_in) * kernel_h * kernel_w;
 		const bool zero_fits = (input_zero >= -128 && input_zero <= 127) || (kernel_h == 1 && kernel_w == 1);
 		const bool fast = (filters_in % 16 == 0) && aligned_to(input, 16) && aligned_to(weights, 16) && k_bytes <= 0x7fffffffu && zero_fits;
-		if (fast && filters_in % 128 == 0)
+		if (fast && kernel_h == 1 && kernel_w == 1 && ep.vectorized && stream_gemm_applies(M, 1, k_bytes))
+		{ /* a 1x1 convolution with a short K row is bound by HBM: the persistent streaming kernel on the [B*H*W, Cin] view */
+			const StreamGemmArgs sg { input, weights, nullptr, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0 };
+			launch_stream_gemm<int8_t>(stream, sg, ep);
+		}
+		else if (fast && filters_in % 128 == 0)
 		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */
 			Im2RowDmaRows a_loader;
 			a_loader.base = reinterpret_cast<const uint8_t*>(input);

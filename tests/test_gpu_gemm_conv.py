@@ -106,6 +106,30 @@ def test_gemm_ex_epilogue(ctx, dtype, act):
         assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("k_bytes", [128, 256, 512])
+@pytest.mark.parametrize("M,N", [(33001, 256), (32800, 100), (40000, 64), (33000, 28), (32769, 384)])
+def test_gemm_ex_streaming_shapes(ctx, dtype, k_bytes, M, N):
+    """gemm_ex with short K rows and many rows of A (1x1 convolutions, dense heads): the persistent streaming kernel with the fused
+    epilogue. All three wavefront layouts (N > 128, > 64, <= 64), column counts that are no multiple of 32, a ragged last row block,
+    more than 256 columns; bias + beta * C + ReLU, and a sigmoid in place."""
+    K = k_bytes // (2 if dtype == "float16" else 4)
+    rng = np.random.default_rng(M + N + k_bytes)
+    A = random_tensor(rng, (M, K), dtype, 0.3)
+    Bm = random_tensor(rng, (N, K), dtype, 0.3)
+    C = random_tensor(rng, (M, N), dtype)
+    bias = random_tensor(rng, (N,), dtype)
+    dA, dB = ml.toDevice(ctx, A), ml.toDevice(ctx, Bm)
+    dD = ml.Tensor((M, N), dtype)
+    dD.setall(ctx, float("nan"))
+    ml.gemm_ex(ctx, dD, 1.1, "n", dA, "t", dB, 0.5, ml.toDevice(ctx, C), ml.toDevice(ctx, bias), "relu")
+    want = O.gemm(A, Bm, alpha=1.1, beta=0.5, C=C, bias=bias, act=O.RELU)
+    assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype]
+    dD = ml.toDevice(ctx, C)
+    ml.gemm_ex(ctx, dD, 1.0, "n", dA, "t", dB, 1.0, dD, None, "sigmoid")
+    assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, alpha=1.0, beta=1.0, C=C, act=O.SIGMOID)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("tag,dtype", [("f32", "float32"), ("f16", "float16")])
 def test_reference_fixtures(ctx, golden, tag, dtype):
     g = golden

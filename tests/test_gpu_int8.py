@@ -24,7 +24,8 @@ def init_for_test_int8(shape, shift):
     return ((v + 128) % 256 - 128).astype(np.int8).reshape(shape)
 
 
-@pytest.mark.parametrize("shape", [(75, 44, 36), (1716, 44, 36), (130, 70, 64), (300, 256, 2304), (33, 5, 20), (64, 64, 16)])
+@pytest.mark.parametrize("shape", [(75, 44, 36), (1716, 44, 36), (130, 70, 64), (300, 256, 2304), (33, 5, 20), (64, 64, 16),
+                                   (33001, 256, 256), (40000, 72, 128), (32900, 132, 512)])
 def test_int8_gemm_exact(ctx, shape):
     M, N, K = shape
     rng = np.random.default_rng(M)
