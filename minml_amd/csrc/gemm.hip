@@ -124,11 +124,12 @@ namespace mlhip
 		 * the Winograd products with a plain 16-byte store, everything else (gemm_ex, 1x1 convolutions, the int8 product) with the
 		 * fused epilogue on 4 consecutive outputs.
 		 */
-		if (fast && stream_gemm_applies(g.M, g.batch, k_bytes) && (g.stride_a != 0 || g.batch == 1))
+		const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR) && (g.N * esize) % 16 == 0
+				&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0) && g.dtype != DTYPE_INT8;
+		if (fast && (g.stride_a != 0 || g.batch == 1)
+				&& (plain ? stream_gemm_plain_applies(g.M, g.batch, k_bytes, esize) : stream_gemm_applies(g.M, g.batch, k_bytes)))
 		{
 			const StreamGemmArgs sg { g.A, g.B, g.D, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a, g.stride_b, g.stride_c };
-			const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR) && (g.N * esize) % 16 == 0
-					&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0);
 			bool launched = true;
 			if (g.dtype == DTYPE_FLOAT16 && plain)
 				launch_stream_gemm<half_t>(stream, sg, PlainStore { });

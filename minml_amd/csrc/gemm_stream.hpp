@@ -428,6 +428,11 @@ namespace mlhip
 	{
 		return (k_bytes == 128 || k_bytes == 256 || k_bytes == 512) && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256;
 	}
+	/* the plain-store fp16 form is also instantiated for 768-byte rows (384 halfs), whose B operand still fits the registers */
+	inline bool stream_gemm_plain_applies(int M, int batch, size_t k_bytes, int element_size)
+	{
+		return stream_gemm_applies(M, batch, k_bytes) || (element_size == 2 && k_bytes == 768 && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256);
+	}
 	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue>
 	inline void launch_stream_gemm_as(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
 	{
@@ -481,6 +486,13 @@ namespace mlhip
 			case 512:
 				launch_stream_gemm_kb<T, 512>(stream, g, epilogue);
 				break;
+			case 768:
+				if constexpr (std::is_same<Epilogue, PlainStore>::value && sizeof(T) == 2)
+				{
+					launch_stream_gemm_kb<T, 768>(stream, g, epilogue);
+					break;
+				}
+				[[fallthrough]];
 			default:
 				fail_logic("HIP backend: streaming GEMM: unsupported K row length");
 		}

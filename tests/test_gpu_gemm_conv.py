@@ -68,6 +68,20 @@ def test_gemm_batched_nt_streaming_shapes(ctx, dtype, shape):
     assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm[0])) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype,K", [("float16", 384), ("float16", 64), ("float16", 128), ("float32", 32), ("float32", 64)])
+@pytest.mark.parametrize("shape", [(36, 1000, 384), (9, 4100, 72), (36, 950, 128)])
+def test_gemm_batched_nt_streaming_other_row_lengths(ctx, dtype, K, shape):
+    """The same kernel for K rows of 128, 256 and 768 bytes (Winograd products at 64, 128 and 384 channels)."""
+    bt, M, N = shape
+    rng = np.random.default_rng(sum(shape) + K)
+    A = random_tensor(rng, (bt, M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (bt, N, K), dtype, 0.5)
+    dC = ml.Tensor((bt, M, N), dtype)
+    dC.setall(ctx, float("nan"))
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.0, 0.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_gemm_batched_broadcast_and_beta(ctx, dtype):
     rng = np.random.default_rng(5)
