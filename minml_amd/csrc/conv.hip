@@ -90,14 +90,11 @@ namespace
 		const int pad = (kernel_size - 1) / 2;
 		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
 		{
-			const int c = static_cast<int>(gid % vecs_per_pixel);
-			size_t rest = gid / vecs_per_pixel;
-			const int tap = static_cast<int>(rest % taps);
-			rest /= taps;
-			const int w = static_cast<int>(rest % width);
-			rest /= width;
-			const int h = static_cast<int>(rest % height);
-			const int b = static_cast<int>(rest / height);
+			int c, tap, w, h;
+			size_t rest = split_index(gid, vecs_per_pixel, c);
+			rest = split_index(rest, taps, tap);
+			rest = split_index(rest, width, w);
+			const int b = static_cast<int>(split_index(rest, height, h));
 			const int i = tap / kernel_size, j = tap % kernel_size;
 			const int x = h - pad + (invert ? (kernel_size - 1 - i) : i);
 			const int y = w - pad + (invert ? (kernel_size - 1 - j) : j);

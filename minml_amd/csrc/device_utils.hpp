@@ -152,6 +152,24 @@ namespace mlhip
 			}
 	};
 
+	/*
+	 * quotient and remainder of a flat index by a 32-bit extent. 64-bit integer division is a long instruction sequence on this
+	 * hardware and dominates a bandwidth-bound kernel that does one per 16 bytes; indices below 2^32 take the 32-bit form.
+	 */
+	__device__ __forceinline__ size_t split_index(size_t index, int extent, int &remainder)
+	{
+		if ((index >> 32) == 0)
+		{
+			const uint32_t i = static_cast<uint32_t>(index), d = static_cast<uint32_t>(extent);
+			const uint32_t q = i / d;
+			remainder = static_cast<int>(i - q * d);
+			return q;
+		}
+		const size_t q = index / static_cast<size_t>(extent);
+		remainder = static_cast<int>(index - q * static_cast<size_t>(extent));
+		return q;
+	}
+
 	/* activations of the reference (src/backend/cpu/common_math.hpp:40-55, src/backend/cpu/def_misc_kernels.cpp:52-72) */
 	__device__ __forceinline__ float activate(int act, float x)
 	{

@@ -26,12 +26,15 @@ namespace
 		const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
 		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
 		{
-			const int col = static_cast<int>(gid % groups) * VEC;
-			const size_t offset = (gid / groups) * last_dim + col;
+			const size_t offset = gid * VEC; /* rows are contiguous and last_dim == groups * VEC */
 			Vec<T, VEC> vx, vb, vy;
 			vx.load(x + offset);
 			if (bias != nullptr)
-				vb.load(bias + col);
+			{
+				int group;
+				split_index(gid, groups, group);
+				vb.load(bias + group * VEC);
+			}
 			else
 				vb.zero();
 			if (beta != 0.0f)
@@ -83,12 +86,22 @@ namespace
 		}
 	}
 
-	template<typename DstT, typename SrcT>
+	/* VEC elements per thread and step: 8 gives one 16-byte access on the fp16 side and two on the fp32 side. */
+	template<typename DstT, typename SrcT, int VEC>
 	__global__ __launch_bounds__(256) void kernel_convert(DstT *dst, const SrcT *src, size_t elements)
 	{
+		const size_t total = elements / VEC;
 		const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
-		for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < elements; i += stride)
-			Storage<DstT>::store(dst + i, Storage<SrcT>::load(src + i));
+		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
+		{
+			Vec<SrcT, VEC> in;
+			in.load(src + gid * VEC);
+			Vec<DstT, VEC> out;
+#pragma unroll
+			for (int e = 0; e < VEC; e++)
+				out.v[e] = in.v[e];
+			out.store(dst + gid * VEC);
+		}
 	}
 
 	template<typename T>
@@ -104,10 +117,35 @@ namespace
 		const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
 		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
 		{
-			const size_t i = gid / last_dim;
-			const int j = static_cast<int>(gid % last_dim);
+			int j;
+			const size_t i = split_index(gid, last_dim, j);
 			const uint32_t word = src[i * words + j / 32];
 			dst[gid] = one_or_zero<T>((word >> (j % 32)) & 1u);
+		}
+	}
+	/*
+	 * last_dim a multiple of GROUP (a power of two up to 32, GROUP * sizeof(T) == 16 where the type allows): one thread
+	 * expands GROUP consecutive bits of one word and writes them with 16-byte stores.
+	 */
+	template<typename T, int GROUP>
+	__global__ __launch_bounds__(256) void kernel_unpack_input_grouped(T *dst, const uint32_t *src, size_t first_dim, int last_dim)
+	{
+		typedef T vt __attribute__((ext_vector_type(GROUP)));
+		const int words = (last_dim + 31) / 32;
+		const int groups = last_dim / GROUP;
+		const size_t total = first_dim * groups;
+		const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
+		{
+			int group;
+			const size_t i = split_index(gid, groups, group);
+			const int j = group * GROUP;
+			const uint32_t bits = src[i * words + j / 32] >> (j % 32);
+			vt out;
+#pragma unroll
+			for (int e = 0; e < GROUP; e++)
+				out[e] = one_or_zero<T>((bits >> e) & 1u);
+			*reinterpret_cast<vt*>(dst + i * last_dim + j) = out;
 		}
 	}
 
@@ -121,13 +159,41 @@ namespace
 		return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 	}
 
+	template<typename DstT, typename SrcT>
+	void launch_convert(hipStream_t stream, DstT *dst, const SrcT *src, size_t elements)
+	{
+		constexpr int VEC = 8;
+		const size_t body = (aligned_to(dst, VEC * sizeof(DstT)) && aligned_to(src, VEC * sizeof(SrcT))) ? (elements / VEC) * VEC : 0;
+		if (body > 0)
+			hipLaunchKernelGGL((kernel_convert<DstT, SrcT, VEC>), dim3(grid_for(body / VEC)), dim3(256), 0, stream, dst, src, body);
+		if (body < elements)
+			hipLaunchKernelGGL((kernel_convert<DstT, SrcT, 1>), dim3(grid_for(elements - body)), dim3(256), 0, stream, dst + body, src + body,
+					elements - body);
+	}
+	template<typename T>
+	void launch_unpack_input(hipStream_t stream, T *dst, const uint32_t *src, size_t first, int last)
+	{
+		constexpr int GROUP = (sizeof(T) >= 4) ? 4 : static_cast<int>(16 / sizeof(T));
+		if (last % GROUP == 0 && aligned_to(dst, GROUP * sizeof(T)))
+			hipLaunchKernelGGL((kernel_unpack_input_grouped<T, GROUP>), dim3(grid_for(first * (last / GROUP))), dim3(256), 0, stream, dst, src, first,
+					last);
+		else
+			hipLaunchKernelGGL(kernel_unpack_input<T>, dim3(grid_for(first * last)), dim3(256), 0, stream, dst, src, first, last);
+	}
+
 	template<typename T>
 	void launch_add_bias_act(hipStream_t stream, float alpha, const mlTensor_t &x, const mlTensor_t &b, float beta, mlTensor_t &y, int act)
 	{
 		const int last = last_dim(x);
 		const size_t first = volume(x) / last;
-		const bool vec4 = (last % 4 == 0) && aligned_to(x.data, 4 * sizeof(T)) && aligned_to(y.data, 4 * sizeof(T)) && aligned_to(b.data, 4 * sizeof(T));
-		if (vec4)
+		constexpr int WIDE = 16 / static_cast<int>(sizeof(T)); /* elements of one 16-byte access */
+		const auto fits = [&](int vec) {
+			return (last % vec == 0) && aligned_to(x.data, vec * sizeof(T)) && aligned_to(y.data, vec * sizeof(T)) && aligned_to(b.data, vec * sizeof(T));
+		};
+		if (WIDE > 4 && fits(WIDE))
+			hipLaunchKernelGGL((kernel_add_bias_act<T, WIDE>), dim3(grid_for(first * (last / WIDE))), dim3(256), 0, stream, beta, ptr<T>(y), alpha,
+					ptr<const T>(x), ptr<const T>(b), first, last, act);
+		else if (fits(4))
 			hipLaunchKernelGGL((kernel_add_bias_act<T, 4>), dim3(grid_for(first * (last / 4))), dim3(256), 0, stream, beta, ptr<T>(y), alpha, ptr<const T>(x),
 					ptr<const T>(b), first, last, act);
 		else
@@ -140,9 +206,15 @@ namespace
 			mlTensor_t &y)
 	{
 		const size_t elements = volume(y);
-		const bool vec4 = (elements % 4 == 0) && aligned_to(x1.data, 4 * sizeof(T)) && aligned_to(x2.data, 4 * sizeof(T))
-				&& aligned_to(x3.data, 4 * sizeof(T)) && aligned_to(y.data, 4 * sizeof(T));
-		if (vec4)
+		constexpr int WIDE = 16 / static_cast<int>(sizeof(T)); /* elements of one 16-byte access */
+		const auto fits = [&](int vec) {
+			return (elements % vec == 0) && aligned_to(x1.data, vec * sizeof(T)) && aligned_to(x2.data, vec * sizeof(T))
+					&& aligned_to(x3.data, vec * sizeof(T)) && aligned_to(y.data, vec * sizeof(T));
+		};
+		if (WIDE > 4 && fits(WIDE))
+			hipLaunchKernelGGL((kernel_axpy3<T, WIDE>), dim3(grid_for(elements / WIDE)), dim3(256), 0, stream, a1, ptr<const T>(x1), a2, ptr<const T>(x2),
+					a3, ptr<const T>(x3), beta, ptr<T>(y), elements);
+		else if (fits(4))
 			hipLaunchKernelGGL((kernel_axpy3<T, 4>), dim3(grid_for(elements / 4)), dim3(256), 0, stream, a1, ptr<const T>(x1), a2, ptr<const T>(x2), a3,
 					ptr<const T>(x3), beta, ptr<T>(y), elements);
 		else
@@ -198,13 +270,7 @@ extern "C"
 		no_bias.data = nullptr;
 		no_bias.dtype = x.dtype;
 		no_bias.rank = 0;
-		/* view as [elements / 4, 4] when possible so that the vector path applies */
-		if (flat.dim[0] % 4 == 0)
-		{
-			flat.rank = flat_y.rank = 2;
-			flat.dim[1] = flat_y.dim[1] = 4;
-			flat.dim[0] = flat_y.dim[0] = flat.dim[0] / 4;
-		}
+		/* one row of all elements: the widest vector form that divides the length applies */
 		hip_add_bias_act(context, alpha, flat, no_bias, beta, flat_y, act);
 	}
 	void hip_add_tensors(mlContext_t context, float alpha1, const mlTensor_t x1, float alpha2, const mlTensor_t x2, float alpha3, const mlTensor_t x3,
@@ -246,11 +312,9 @@ extern "C"
 		}
 		const size_t n = static_cast<size_t>(elements);
 		if (src_dtype == DTYPE_FLOAT32 && dst_dtype == DTYPE_FLOAT16)
-			hipLaunchKernelGGL((kernel_convert<half_t, float>), dim3(grid_for(n)), dim3(256), 0, stream_of(context), reinterpret_cast<half_t*>(dst),
-					reinterpret_cast<const float*>(src), n);
+			launch_convert(stream_of(context), reinterpret_cast<half_t*>(dst), reinterpret_cast<const float*>(src), n);
 		else if (src_dtype == DTYPE_FLOAT16 && dst_dtype == DTYPE_FLOAT32)
-			hipLaunchKernelGGL((kernel_convert<float, half_t>), dim3(grid_for(n)), dim3(256), 0, stream_of(context), reinterpret_cast<float*>(dst),
-					reinterpret_cast<const half_t*>(src), n);
+			launch_convert(stream_of(context), reinterpret_cast<float*>(dst), reinterpret_cast<const half_t*>(src), n);
 		else
 			fail_logic("unsupported conversion");
 		MLHIP_CHECK(hipGetLastError());
@@ -262,27 +326,27 @@ extern "C"
 		MLHIP_REQUIRE(dst != nullptr && src != nullptr, "unpack_input: null pointer");
 		const int last = last_dim(shape);
 		const size_t first = volume(shape) / last;
-		const dim3 grid(grid_for(first * last)), block(256);
 		const uint32_t *in = reinterpret_cast<const uint32_t*>(src);
+		const hipStream_t stream = stream_of(context);
 		switch (dst_dtype)
 		{
 			case DTYPE_FLOAT16:
-				hipLaunchKernelGGL(kernel_unpack_input<half_t>, grid, block, 0, stream_of(context), reinterpret_cast<half_t*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<half_t*>(dst), in, first, last);
 				break;
 			case DTYPE_FLOAT32:
-				hipLaunchKernelGGL(kernel_unpack_input<float>, grid, block, 0, stream_of(context), reinterpret_cast<float*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<float*>(dst), in, first, last);
 				break;
 			case DTYPE_UINT8:
-				hipLaunchKernelGGL(kernel_unpack_input<uint8_t>, grid, block, 0, stream_of(context), reinterpret_cast<uint8_t*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<uint8_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT8:
-				hipLaunchKernelGGL(kernel_unpack_input<int8_t>, grid, block, 0, stream_of(context), reinterpret_cast<int8_t*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<int8_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT16:
-				hipLaunchKernelGGL(kernel_unpack_input<int16_t>, grid, block, 0, stream_of(context), reinterpret_cast<int16_t*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<int16_t*>(dst), in, first, last);
 				break;
 			case DTYPE_INT32:
-				hipLaunchKernelGGL(kernel_unpack_input<int32_t>, grid, block, 0, stream_of(context), reinterpret_cast<int32_t*>(dst), in, first, last);
+				launch_unpack_input(stream, reinterpret_cast<int32_t*>(dst), in, first, last);
 				break;
 			default:
 				fail_logic("HIP backend: unpack_input: unsupported destination type");

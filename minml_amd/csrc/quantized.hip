@@ -31,8 +31,9 @@ namespace
 		const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
 		for (size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; gid < total; gid += stride)
 		{
-			const int m = static_cast<int>(gid / groups);
-			const int n = static_cast<int>(gid % groups) * 4;
+			int group;
+			const int m = static_cast<int>(split_index(gid, groups, group));
+			const int n = group * 4;
 			const int32_t *src = input + static_cast<size_t>(m) * last_dim + n;
 			int acc[4] = { 0, 0, 0, 0 };
 			if (epilogue.vectorized)

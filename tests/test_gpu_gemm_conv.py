@@ -284,3 +284,30 @@ def test_convert_and_unpack(ctx, golden):
         d = ml.Tensor((3, 5, 40), code)
         ml.unpackInput(ctx, d, ml.toDevice(ctx, g["up_packed"].view(np.int32), "int32"))
         assert mismatches(d.copyToHost(ctx), g[key]) == 0
+
+
+@pytest.mark.parametrize("last", [32, 40, 48, 7, 100])
+@pytest.mark.parametrize("dtype", ["float16", "float32"])
+def test_unpack_input_vector_and_scalar_forms(ctx, last, dtype):
+    """Row lengths that take the 16-byte-store form (multiples of 8 halfs / 4 floats) and ones that do not, bit for bit."""
+    rng = np.random.default_rng(last)
+    words = (last + 31) // 32
+    packed = rng.integers(0, 2 ** 32, size=(6 * 15 * 15, words), dtype=np.uint64).astype(np.uint32)
+    d = ml.Tensor((6, 15, 15, last), dtype)
+    ml.unpackInput(ctx, d, ml.toDevice(ctx, packed.view(np.int32), "int32"))
+    want = O.unpack_input(packed, (6, 15, 15, last), O.FLOAT16 if dtype == "float16" else O.FLOAT32)
+    assert mismatches(d.copyToHost(ctx), want) == 0
+
+
+@pytest.mark.parametrize("elements", [8, 4099, 1 << 20])
+def test_convert_type_vector_body_and_tail(ctx, elements):
+    """Lengths with and without a scalar tail after the 8-element vector body; both directions, bit for bit."""
+    rng = np.random.default_rng(elements)
+    src = (rng.standard_normal(elements) * 50.0).astype(np.float32)
+    dst = ml.Tensor((elements,), "float16")
+    ml.convertType(ctx, dst, ml.toDevice(ctx, src))
+    got = dst.copyToHost(ctx)
+    assert mismatches(got, O.to_half(src)) == 0
+    back = ml.Tensor((elements,), "float32")
+    ml.convertType(ctx, back, dst)
+    assert np.array_equal(back.copyToHost(ctx), O.from_half(got))
