@@ -147,6 +147,18 @@ extern "C"
 			float beta, mlTensor_t y);
 	void hip_scale_tensor(mlContext_t context, float alpha, mlTensor_t x); /* x *= alpha (reference: cuda_backend.h:295) */
 
+	/* ---- steps after the path: policy softmax, pooling before a value head, batch normalisation in inference mode and its folding
+	 *      into the preceding layer (reference: cuda_backend.h:127,177-178,185-186,230; arithmetic of the CPU backend where it has one:
+	 *      src/backend/cpu/avx_misc_kernels.cpp:53-112, src/backend/cpu/kernels/pooling_and_scaling.cpp:142-180,
+	 *      src/backend/cpu/normalization.cpp:296-343; batchnorm_inference follows src/backend/cuda/kernels/batchnorm.cu:57-104,
+	 *      its CPU dispatch being commented out in src/core/math.cpp:722-737). fp16 and fp32. ---- */
+	void hip_softmax_forward(mlContext_t context, mlDataType_t dtype, mlShape_t shape, void *output, const void *input); /* rows of the last dim; in place allowed */
+	void hip_global_average_pooling_forward(mlContext_t context, float alpha, const mlTensor_t x, float beta, mlTensor_t y); /* [B,H,W,C] -> [B,C] */
+	void hip_batchnorm_inference(mlContext_t context, float alpha, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, const mlTensor_t avg_var,
+			float beta, mlTensor_t y, mlActivationType_t act); /* avg_var fp32 [2, C]: means, variances; w / b may be empty */
+	void hip_fold_batchnorm(mlContext_t context, mlTensor_t layer_weights, mlTensor_t layer_bias, const mlTensor_t bn_weights, const mlTensor_t bn_bias,
+			const mlTensor_t bn_avg_var); /* in place; rank-3 weights are depthwise (channels last), others channels first */
+
 	/* ---- additions with no counterpart in the reference ABI ----
 	 * hip_quantized_conv_forward: the whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 (int8 implicit GEMM with
 	 * zero-point padding, int32 accumulation, per-channel scale + bias, optional int8 residual, activation, requantisation)

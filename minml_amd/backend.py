@@ -95,6 +95,10 @@ SIGNATURES = {
     "activation_forward": (None, [_vp, _f, _T, _f, _T, _i]),
     "add_tensors": (None, [_vp, _f, _T, _f, _T, _f, _T, _f, _T]),
     "scale_tensor": (None, [_vp, _f, _T]),
+    "softmax_forward": (None, [_vp, _i, _S, _vp, _vp]),
+    "global_average_pooling_forward": (None, [_vp, _f, _T, _f, _T]),
+    "batchnorm_inference": (None, [_vp, _f, _T, _T, _T, _T, _f, _T, _i]),
+    "fold_batchnorm": (None, [_vp, _T, _T, _T, _T, _T]),
     "quantized_conv_forward": (None, [_vp, _S, _S, _vp, _Q, _vp, _vp, _vp, _i, _vp, _Q, _vp, _Q, _i]),
     "get_stream": (_vp, [_vp]),
 }

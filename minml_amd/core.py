@@ -475,3 +475,35 @@ def unpackInput(context, dst, src):
     words = (dst.lastDim() + 31) // 32
     _require(src.sizeInBytes() >= (dst.volume() // dst.lastDim()) * words * 4, "packed input too small")
     B.fn("unpack_input")(context.handle, dst.shape_desc(), dst.dtype, dst.ptr, src.ptr)
+
+
+def softmaxForward(context, output, input):
+    """Row-wise softmax over the last dimension; output may be the input (reference: src/core/math.cpp:1013-1029)."""
+    _require(_same_dtype(input, output) and input.volume() == output.volume(), "shape / dtype mismatch")
+    _launch("softmax_forward", context.handle, input.dtype, input.shape_desc(), output.ptr, input.ptr)
+
+
+def globalAveragePoolingForward(context, alpha, input, beta, output):
+    """[B, H, W, C] -> [B, C]: alpha * mean over the pixels + beta * output (reference: src/core/math.cpp:515-531)."""
+    _require(len(input.shape) == 4 and len(output.shape) == 2, "input must be [B, H, W, C] and output [B, C]")
+    _require(input.shape[0] == output.shape[0] and input.shape[3] == output.shape[1] and _same_dtype(input, output), "shape / dtype mismatch")
+    _launch("global_average_pooling_forward", context.handle, alpha, input.desc(), beta, output.desc())
+
+
+def batchnormInference(context, alpha, input, weights, bias, avg_var, beta, output, act="linear"):
+    """alpha * act((x - mean) * gamma / sqrt(var + 1e-6) + bias) + beta * output; avg_var fp32 [2, C] (reference: src/core/math.cpp:722-737)."""
+    _require(_same_dtype(input, weights, bias, output) and input.volume() == output.volume(), "shape / dtype mismatch")
+    _require(avg_var.dtype == B.DTYPE_FLOAT32 and avg_var.volume() == 2 * input.lastDim(), "statistics must be fp32 [2, C]")
+    for t in (weights, bias):
+        _require(t is None or t.isEmpty() or t.volume() == input.lastDim(), "gamma / bias must be [C]")
+    _launch("batchnorm_inference", context.handle, alpha, input.desc(), _desc(weights), _desc(bias), avg_var.desc(), beta, output.desc(), act_of(act))
+
+
+def foldBatchnorm(context, layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
+    """Folds a batch normalisation into the preceding layer's weights and bias, in place (reference: src/core/math.cpp:786-802, which
+    also synchronises with the context afterwards)."""
+    channels = layer_weights.shape[-1] if len(layer_weights.shape) == 3 else layer_weights.shape[0]
+    _require(_same_dtype(layer_weights, layer_bias, bn_weights, bn_bias) and layer_bias.volume() == channels, "shape / dtype mismatch")
+    _require(bn_avg_var.dtype == B.DTYPE_FLOAT32 and bn_avg_var.volume() == 2 * channels, "statistics must be fp32 [2, channels]")
+    B.fn("fold_batchnorm")(context.handle, layer_weights.desc(), layer_bias.desc(), _desc(bn_weights), _desc(bn_bias), bn_avg_var.desc())
+    context.synchronize()

@@ -42,7 +42,6 @@ MLHIP_STUB(cuda_quantized_depthwise_conv_forward)
 /* pooling and scaling */
 MLHIP_STUB(cuda_average_pooling_forward)
 MLHIP_STUB(cuda_average_pooling_backward)
-MLHIP_STUB(cuda_global_average_pooling_forward)
 MLHIP_STUB(cuda_global_average_pooling_backward)
 MLHIP_STUB(cuda_channel_scaling_forward)
 MLHIP_STUB(cuda_channel_scaling_backward)
@@ -53,11 +52,9 @@ MLHIP_STUB(cuda_spatial_scaling_backward)
 MLHIP_STUB(cuda_learnable_scaling_forward)
 MLHIP_STUB(cuda_learnable_scaling_backward)
 /* normalisation */
-MLHIP_STUB(cuda_batchnorm_inference)
 MLHIP_STUB(cuda_batchnorm_forward)
 MLHIP_STUB(cuda_batchnorm_backward)
 MLHIP_STUB(cuda_batchnorm_update)
-MLHIP_STUB(cuda_fold_batchnorm)
 MLHIP_STUB(cuda_layernorm_forward)
 MLHIP_STUB(cuda_layernorm_backward)
 MLHIP_STUB(cuda_rmsnorm_forward)
@@ -81,7 +78,6 @@ MLHIP_STUB(cuda_moe_forward)
 MLHIP_STUB(cuda_moe_backward)
 /* backward passes, softmax, tensor helpers */
 MLHIP_STUB(cuda_activation_backward)
-MLHIP_STUB(cuda_softmax_forward)
 MLHIP_STUB(cuda_softmax_backward)
 MLHIP_STUB(cuda_fused_act_bias_copy_backward)
 MLHIP_STUB(cuda_emulate_low_precision)

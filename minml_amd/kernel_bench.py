@@ -8,7 +8,7 @@ achieved fraction of that peak.
 
 Groups: winograd (transforms and batched GEMM at the residual-network shapes), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
 channels 64..384, kernels 1 / 3 / 5, bias + residual + ReLU), int8 (quantised 3x3 convolution at 256 channels and its three-call form),
-misc (im2row, element-wise neighbours).
+misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode).
 """
 import argparse
 import json
@@ -183,15 +183,39 @@ class Bench:
             t.free()
 
 
+    def heads(self):
+        ctx, rng = self.ctx, self.rng
+        batch, board, chans, dtype, s = 1024, 15, 256, "float16", 2
+        pix = batch * board * board
+        x = _random(ctx, (batch, board, board, chans), dtype, rng)
+        y = ml.Tensor((batch, board, board, chans), dtype)
+        pooled = ml.Tensor((batch, chans), dtype)
+        gamma = _random(ctx, (chans,), dtype, rng, 0.1)
+        bias = _random(ctx, (chans,), dtype, rng, 0.1)
+        stats = ml.toDevice(ctx, np.stack([rng.standard_normal(chans), rng.random(chans) + 0.5]).astype(np.float32), "float32")
+        shape = "cfg2 [1024,15,15,256] f16"
+        self.row("heads", "global_average_pooling_forward", shape, lambda: ml.globalAveragePoolingForward(ctx, 1.0, x, 0.0, pooled),
+                 s * (pix * chans + batch * chans))
+        self.row("heads", "batchnorm_inference (relu)", shape, lambda: ml.batchnormInference(ctx, 1.0, x, gamma, bias, stats, 0.0, y, "relu"),
+                 s * 2 * pix * chans)
+        logits = _random(ctx, (batch, board * board), dtype, rng, 3.0)
+        policy = ml.Tensor((batch, board * board), dtype)
+        self.row("heads", "softmax_forward (policy)", "cfg2 [1024,225] f16", lambda: ml.softmaxForward(ctx, policy, logits), s * 2 * batch * board * board)
+        many = _random(ctx, (pix, chans), dtype, rng, 3.0)
+        self.row("heads", "softmax_forward (256 columns)", "[230400,256] f16", lambda: ml.softmaxForward(ctx, y, many), s * 2 * pix * chans)
+        for t in (x, y, pooled, gamma, bias, stats, logits, policy, many):
+            t.free()
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
-    for group in ("winograd", "conv", "int8", "misc"):
+    for group in ("winograd", "conv", "int8", "misc", "heads"):
         if args.group in ("all", group):
             getattr(bench, group)()
     if args.json:

@@ -65,6 +65,10 @@ def lib():
         _lib.oracle_add_bias_act.argtypes = [_i, _sz, _i, _c_void_p, _c_void_p, _c_void_p, _i]
         _lib.oracle_add_tensors.argtypes = [_i, _sz, _f, _c_void_p, _f, _c_void_p, _f, _c_void_p, _f, _c_void_p]
         _lib.oracle_unpack_input.argtypes = [_i, _sz, _i, _c_void_p, _c_void_p]
+        _lib.oracle_softmax_forward.argtypes = [_i, _sz, _i, _c_void_p, _c_void_p]
+        _lib.oracle_global_average_pooling_forward.argtypes = [_i, _i, _i, _i, _f, _c_void_p, _f, _c_void_p]
+        _lib.oracle_batchnorm_inference.argtypes = [_i, _sz, _i, _f, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _f, _c_void_p, _i]
+        _lib.oracle_fold_batchnorm.argtypes = [_i, _i, _i, _i, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]
     return _lib
 
 
@@ -234,11 +238,65 @@ def unpack_input(packed, shape, dtype):
     return out
 
 
+def softmax_forward(x):
+    """Row-wise softmax over the last dimension."""
+    x = _c(x)
+    out = np.empty_like(x)
+    lib().oracle_softmax_forward(dtype_code(x), x.size // x.shape[-1], x.shape[-1], _p(out), _p(x))
+    return out
+
+
+def global_average_pooling_forward(x, alpha=1.0, beta=0.0, y=None):
+    """[B, H, W, C] -> [B, C]: alpha * mean over the pixels + beta * y."""
+    x = _c(x)
+    b, h, w, c = x.shape
+    out = np.zeros((b, c), x.dtype) if y is None else np.array(y, copy=True, order="C")
+    lib().oracle_global_average_pooling_forward(dtype_code(x), b, h * w, c, alpha, _p(x), beta, _p(out))
+    return out
+
+
+def batchnorm_inference(x, gamma, bias, avg_var, act=LINEAR, alpha=1.0, beta=0.0, y=None):
+    """alpha * act((x - mean) * gamma / sqrt(var + 1e-6) + bias) + beta * y; avg_var fp32 [2, C]."""
+    x, gamma, bias = _c(x), _c(gamma), _c(bias)
+    avg_var = _c(avg_var, np.float32)
+    out = np.zeros_like(x) if y is None else np.array(y, copy=True, order="C")
+    lib().oracle_batchnorm_inference(dtype_code(x), x.size // x.shape[-1], x.shape[-1], alpha, _p(x), _p(gamma), _p(bias), _p(avg_var), beta,
+                                     _p(out), act)
+    return out
+
+
+def fold_batchnorm(layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
+    """Returns (weights, bias) with the batch normalisation folded in. Rank-3 weights are depthwise (channels last)."""
+    w = np.array(layer_weights, copy=True, order="C")
+    b = np.array(layer_bias, copy=True, order="C")
+    last = w.ndim == 3
+    channels = w.shape[-1] if last else w.shape[0]
+    lib().oracle_fold_batchnorm(dtype_code(w), channels, w.size // channels, int(last), _p(w), _p(b), _p(_c(bn_weights)), _p(_c(bn_bias)),
+                                _p(_c(bn_avg_var, np.float32)))
+    return w, b
+
+
 # ---------------------------------------------------------------------------------------------------------------------------
 # the reference's own CPU backend, compiled from its sources by `make -C oracle ref` (present only where that was built)
 # ---------------------------------------------------------------------------------------------------------------------------
 class _Shape(ctypes.Structure):
     _fields_ = [("rank", _i), ("dim", _i * 6)]
+
+
+class _Tensor(ctypes.Structure):
+    _fields_ = [("data", _c_void_p), ("dtype", _i), ("rank", _i), ("dim", _i * 6)]
+
+
+def _tensor(a):
+    t = _Tensor()
+    if a is None:
+        return t
+    t.data = a.ctypes.data
+    t.dtype = dtype_code(a)
+    t.rank = a.ndim
+    for k, d in enumerate(a.shape):
+        t.dim[k] = int(d)
+    return t
 
 
 def _shape(*dims):
@@ -267,6 +325,9 @@ class Reference:
         L.cpu_add_bias_act.argtypes = [_c_void_p, _i, _Shape, _c_void_p, _c_void_p, _c_void_p, _i]
         L.cpu_unpack_input.argtypes = [_c_void_p, _Shape, _i, _c_void_p, _c_void_p]
         L.cpu_convert_type.argtypes = [_c_void_p, _c_void_p, _i, _c_void_p, _i, _i]
+        L.cpu_softmax_forward.argtypes = [_c_void_p, _i, _Shape, _c_void_p, _c_void_p]
+        L.cpu_global_average_pooling_forward.argtypes = [_c_void_p, _f, _Tensor, _f, _Tensor]
+        L.cpu_fold_batchnorm.argtypes = [_c_void_p, _Tensor, _Tensor, _Tensor, _Tensor, _Tensor]
         self.ctx = L.cpu_create_context()
 
     @staticmethod
@@ -355,6 +416,26 @@ class Reference:
         out = np.zeros(x.shape, np_dtype(dst_dtype))
         self.lib.cpu_convert_type(self.ctx, _p(out), dst_dtype, _p(x), dtype_code(x), x.size)
         return out
+
+    def softmax_forward(self, x):
+        x = _c(x)
+        out = np.zeros_like(x)
+        self.lib.cpu_softmax_forward(self.ctx, dtype_code(x), _shape(x.size // x.shape[-1], x.shape[-1]), _p(out), _p(x))
+        return out
+
+    def global_average_pooling_forward(self, x):
+        x = _c(x)
+        out = np.zeros((x.shape[0], x.shape[3]), x.dtype)
+        self.lib.cpu_global_average_pooling_forward(self.ctx, 1.0, _tensor(x), 0.0, _tensor(out))
+        return out
+
+    def fold_batchnorm(self, layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
+        """fp32 only (the reference reads every argument as float)."""
+        w = np.array(layer_weights, dtype=np.float32, copy=True, order="C")
+        b = np.array(layer_bias, dtype=np.float32, copy=True, order="C")
+        g, bb, st = _c(bn_weights, np.float32), _c(bn_bias, np.float32), _c(bn_avg_var, np.float32)
+        self.lib.cpu_fold_batchnorm(self.ctx, _tensor(w), _tensor(b), _tensor(g), _tensor(bb), _tensor(st))
+        return w, b
 
 
 _ref = None

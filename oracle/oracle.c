@@ -633,3 +633,109 @@ void oracle_unpack_input(int dtype, size_t first_dim, int last_dim, void *dst, c
 			}
 		}
 }
+
+/* ------------------------------------------------------------------------------------------------------------------------
+ * heads and glue after the convolution trunk
+ * ---------------------------------------------------------------------------------------------------------------------- */
+/* src/backend/cpu/avx_misc_kernels.cpp:81-112 (kernel_softmax; the 3-column form at :53-79 is the same arithmetic): row maximum,
+ * exp(x - max) summed in column order, every exponent multiplied by 1 / sum. */
+void oracle_softmax_forward(int dtype, size_t first_dim, int last_dim, void *output, const void *input)
+{
+	float *row = (float*) malloc(sizeof(float) * (size_t) last_dim);
+	for (size_t i = 0; i < first_dim; i++)
+	{
+		const size_t base = i * (size_t) last_dim;
+		for (int j = 0; j < last_dim; j++)
+			row[j] = load_as_float(input, base + j, dtype);
+		float max_value = row[0];
+		for (int j = 0; j < last_dim; j++)
+			max_value = fmaxf(max_value, row[j]);
+		float sum = 0.0f;
+		for (int j = 0; j < last_dim; j++)
+		{
+			row[j] = expf(row[j] - max_value);
+			sum += row[j];
+		}
+		const float scale = 1.0f / sum;
+		for (int j = 0; j < last_dim; j++)
+			store_from_float(output, base + j, dtype, row[j] * scale);
+	}
+	free(row);
+}
+/* src/backend/cpu/kernels/pooling_and_scaling.cpp:142-180 with the SIMD kernels of avx_kernels.cpp:303-560: per (image, channel) the
+ * pixels are summed in row-major order in fp32 and the sum is multiplied by 1.0f / (height * width). alpha and beta follow the
+ * device form (src/backend/cuda/kernels/global_pooling.cu:28-70): y = alpha * mean + beta * y; the CPU entry point only accepts 1, 0. */
+void oracle_global_average_pooling_forward(int dtype, int batch, int hw, int channels, float alpha, const void *input, float beta, void *output)
+{
+	const float inv = 1.0f / (float) hw;
+	/* pooling_and_scaling.cpp:61-92,156-176 on a host with AVX: the widest vector kernel whose step fits the channel count (64 or 8
+	 * columns; 32 or 4 for fp32 through the SSE2 kernels) takes whole steps and multiplies the sum by 1 / hw; what is left goes column
+	 * by column through the scalar kernel, which divides the sum by hw (kernels/def_kernels.cpp:40-54). */
+	int step = 1;
+	if (channels >= 64)
+		step = 64;
+	else if (channels >= 8)
+		step = 8;
+	else if (channels >= 4 && dtype == ORACLE_FLOAT32)
+		step = 4;
+	const int vector_channels = (step > 1) ? (channels / step) * step : 0;
+	for (int b = 0; b < batch; b++)
+		for (int c = 0; c < channels; c++)
+		{
+			float acc = 0.0f;
+			for (int p = 0; p < hw; p++)
+				acc += load_as_float(input, ((size_t) b * hw + p) * channels + c, dtype);
+			const size_t o = (size_t) b * channels + c;
+			float y = (c < vector_channels) ? acc * inv : acc / (float) hw;
+			if (alpha != 1.0f)
+				y *= alpha;
+			if (beta != 0.0f)
+				y += beta * load_as_float(output, o, dtype);
+			store_from_float(output, o, dtype, y);
+		}
+}
+/* src/backend/cuda/kernels/batchnorm.cu:57-104: scale = gamma / sqrt(variance + 1e-6), shift = -mean * scale + beta_bn;
+ * y = alpha * act(x * scale + shift) + beta * y. avg_var is fp32 [2, last_dim] (means, then variances); gamma / bias have the
+ * tensor's type and may be NULL (1 and 0). The CPU dispatch of this entry point is commented out (src/core/math.cpp:722-737). */
+void oracle_batchnorm_inference(int dtype, size_t first_dim, int last_dim, float alpha, const void *input, const void *gamma, const void *bias,
+		const float *avg_var, float beta, void *output, int act)
+{
+	for (size_t i = 0; i < first_dim; i++)
+		for (int j = 0; j < last_dim; j++)
+		{
+			const float g = (gamma != NULL) ? load_as_float(gamma, j, dtype) : 1.0f;
+			const float b = (bias != NULL) ? load_as_float(bias, j, dtype) : 0.0f;
+			const float scale = g / sqrtf(avg_var[last_dim + j] + 1.0e-6f);
+			const float mean_scaled = avg_var[j] * scale;
+			const float shift = b - mean_scaled;
+			const size_t o = i * (size_t) last_dim + j;
+			const float xs = load_as_float(input, o, dtype) * scale;
+			float y = activation(act, xs + shift) * alpha;
+			if (beta != 0.0f)
+				y += beta * load_as_float(output, o, dtype);
+			store_from_float(output, o, dtype, y);
+		}
+}
+/* src/backend/cpu/normalization.cpp:296-343 (cpu_fold_batchnorm) / src/backend/cuda/kernels/batchnorm.cu:357-394: channel-first
+ * weights [channels, last] (channels_last == 0) or depthwise weights [first, channels] (channels_last != 0) are scaled by
+ * gamma / sqrt(variance + 1e-6); bias = bias * scale + (-mean * scale + beta_bn). A NULL bn bias counts as 0 (the device form;
+ * the CPU form uses 1 there and is never called that way: src/graph/graph_optimizers.cpp:165-172 always passes the tensor). */
+void oracle_fold_batchnorm(int dtype, int channels, int other, int channels_last, void *layer_weights, void *layer_bias, const void *bn_weights,
+		const void *bn_bias, const float *bn_avg_var)
+{
+	for (int c = 0; c < channels; c++)
+	{
+		const float gamma = (bn_weights != NULL) ? load_as_float(bn_weights, c, dtype) : 1.0f;
+		const float beta = (bn_bias != NULL) ? load_as_float(bn_bias, c, dtype) : 0.0f;
+		const float scale = gamma / sqrtf(bn_avg_var[channels + c] + 1.0e-6f);
+		const float neg_mean_scaled = -bn_avg_var[c] * scale;
+		const float shift = neg_mean_scaled + beta;
+		const float old_bias_scaled = load_as_float(layer_bias, c, dtype) * scale;
+		store_from_float(layer_bias, c, dtype, old_bias_scaled + shift);
+		for (int k = 0; k < other; k++)
+		{
+			const size_t o = channels_last ? ((size_t) k * channels + c) : ((size_t) c * other + k);
+			store_from_float(layer_weights, o, dtype, load_as_float(layer_weights, o, dtype) * scale);
+		}
+	}
+}

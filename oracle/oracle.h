@@ -92,6 +92,18 @@ extern "C"
 	/* src/backend/cpu/dispatcher.cpp:112-123,143-174: bit j of word (i, j/32) -> 1 / 0 */
 	void oracle_unpack_input(int dtype, size_t first_dim, int last_dim, void *dst, const uint32_t *src);
 
+	/* src/backend/cpu/avx_misc_kernels.cpp:53-112: row-wise softmax over [first_dim, last_dim] */
+	void oracle_softmax_forward(int dtype, size_t first_dim, int last_dim, void *output, const void *input);
+	/* src/backend/cpu/kernels/pooling_and_scaling.cpp:142-180: [batch, hw, channels] -> [batch, channels], y = alpha * mean + beta * y */
+	void oracle_global_average_pooling_forward(int dtype, int batch, int hw, int channels, float alpha, const void *input, float beta,
+			void *output);
+	/* src/backend/cuda/kernels/batchnorm.cu:57-104: y = alpha * act(x * scale + shift) + beta * y with folded statistics */
+	void oracle_batchnorm_inference(int dtype, size_t first_dim, int last_dim, float alpha, const void *input, const void *gamma,
+			const void *bias, const float *avg_var, float beta, void *output, int act);
+	/* src/backend/cpu/normalization.cpp:296-343: batch normalisation folded into the preceding layer's weights and bias, in place */
+	void oracle_fold_batchnorm(int dtype, int channels, int other, int channels_last, void *layer_weights, void *layer_bias,
+			const void *bn_weights, const void *bn_bias, const float *bn_avg_var);
+
 #ifdef __cplusplus
 }
 #endif

@@ -60,6 +60,23 @@ def main():
         out.update({"cv_x_" + tag: cx, "cv_w_" + tag: cw, "cv_bias_" + tag: cb, "cv_add_" + tag: ca, "cv_rows_" + tag: ref.im2row(cx, 5),
                     "cv_y_" + tag: ref.conv2d_forward(cx, cw, cb, ca, O.RELU)})
         out["ab_y_" + tag] = ref.add_bias_act(cx, conv(init_for_test((8,), 0.3)), O.TANH)
+        # after the trunk: policy softmax (225 logits), win / draw / loss softmax, global average pooling (136 = 2 x 64 + 8 channels: the
+        # reference's vector kernels only; 7 channels: its scalar kernel, which divides by the pixel count instead of multiplying)
+        sx = conv(init_for_test((6, 225), 0.0, 3.0))
+        s3 = conv(init_for_test((5, 3), 1.0, 2.0))
+        px = conv(init_for_test((2, 13, 14, 136), 0.0))
+        p7 = conv(init_for_test((2, 5, 5, 7), 1.0))
+        out.update({"sm_x_" + tag: sx, "sm_y_" + tag: ref.softmax_forward(sx), "sm3_x_" + tag: s3, "sm3_y_" + tag: ref.softmax_forward(s3),
+                    "gap_x_" + tag: px, "gap_y_" + tag: ref.global_average_pooling_forward(px),
+                    "gap7_x_" + tag: p7, "gap7_y_" + tag: ref.global_average_pooling_forward(p7)})
+    # batch normalisation folded into a convolution [10,3,3,6] and into depthwise weights [3,3,12] (the reference folds in fp32 only)
+    for key, wshape, channels in (("fd", (10, 3, 3, 6), 10), ("fd3", (3, 3, 12), 12)):
+        fw, fb = init_for_test(wshape, 0.0), init_for_test((channels,), 1.0)
+        gamma, beta = init_for_test((channels,), 2.0) + np.float32(1.5), init_for_test((channels,), 3.0)
+        stats = np.stack([init_for_test((channels,), 4.0), np.abs(init_for_test((channels,), 5.0)) + np.float32(0.1)])
+        folded_w, folded_b = ref.fold_batchnorm(fw, fb, gamma, beta, stats)
+        out.update({key + "_w": fw, key + "_b": fb, key + "_gamma": gamma, key + "_beta": beta, key + "_stats": stats, key + "_w_out": folded_w,
+                    key + "_b_out": folded_b})
     # bit-plane unpacking and fp32 -> fp16 narrowing
     packed = (np.arange(3 * 5 * 2, dtype=np.uint64) * 2654435761 % (1 << 32)).astype(np.uint32)
     out["up_packed"] = packed

@@ -327,3 +327,67 @@ def test_add_bias_act_and_add_tensors():
     got = O.add_tensors(y, 0.5, x, -2.0, x, 0.0, None, 0.25)
     assert np.allclose(got, 0.5 * x - 2.0 * x + 0.25 * y, atol=1e-6)
     assert np.allclose(values(O.add_tensors(O.to_half(y), 1.0, O.to_half(x), beta=1.0)), x + y, atol=4e-3)
+
+
+def test_softmax_known_answer_and_invariants():
+    """The literal of the reference's own test (test/backend/test_nonlinearity.cpp:22-31, tolerance 1e-4 there), rows that sum to one,
+    invariance under a shift of the whole row, and a closed form for two columns (the logistic function)."""
+    x = np.array([[0.1, -0.9, 2.0, 0.0], [0.3, -1.0, 0.7, -0.1]], np.float32)
+    want = np.array([[0.11162444, 0.04106433, 0.74630924, 0.10100197], [0.29114823, 0.07934714, 0.43434212, 0.19516249]], np.float32)
+    assert np.abs(O.softmax_forward(x) - want).max() <= 1e-6
+    assert np.abs(O.as_float(O.softmax_forward(O.to_half(x))) - want).max() <= 1e-3  # the reference's fp16 tolerance
+    rng = np.random.default_rng(5)
+    z = (rng.standard_normal((9, 225)) * 4).astype(np.float32)
+    y = O.softmax_forward(z)
+    assert np.abs(y.sum(axis=1) - 1.0).max() <= 1e-5 and (y >= 0).all()
+    assert np.abs(O.softmax_forward(z + np.float32(7.5)) - y).max() <= 1e-5
+    exact = np.exp(z.astype(np.float64) - z.max(axis=1, keepdims=True))
+    assert np.abs(y - exact / exact.sum(axis=1, keepdims=True)).max() <= 1e-6
+    two = (rng.standard_normal((50, 2)) * 3).astype(np.float32)
+    logistic = 1.0 / (1.0 + np.exp(-(two[:, 0].astype(np.float64) - two[:, 1])))
+    assert np.abs(O.softmax_forward(two)[:, 0] - logistic).max() <= 1e-6
+
+
+def test_global_average_pooling_against_numpy():
+    """The reference's baseline (test/backend/test_global_pooling.cpp:23-40, tolerance 1e-6 in fp32 / 1e-4 in fp16 there) is a plain mean;
+    alpha and beta follow the device form y = alpha * mean + beta * y."""
+    rng = np.random.default_rng(6)
+    x = rng.standard_normal((4, 13, 14, 36)).astype(np.float32)
+    mean = x.astype(np.float64).mean(axis=(1, 2))
+    assert np.abs(O.global_average_pooling_forward(x) - mean).max() <= 1e-6
+    y0 = rng.standard_normal((4, 36)).astype(np.float32)
+    assert np.abs(O.global_average_pooling_forward(x, 0.5, -2.0, y0) - (0.5 * mean - 2.0 * y0)).max() <= 1e-5
+    xh = O.to_half(x)
+    mean_h = O.from_half(xh).astype(np.float64).mean(axis=(1, 2))
+    assert np.abs(O.as_float(O.global_average_pooling_forward(xh)) - mean_h).max() <= 1e-3
+    ones = np.full((2, 4, 4, 8), 1.25, np.float32)  # 16 pixels: the reciprocal is exact
+    assert np.array_equal(O.global_average_pooling_forward(ones), np.full((2, 8), 1.25, np.float32))
+
+
+def test_batchnorm_inference_and_folding_agree():
+    """Closed form in float64, and the identity that folding relies on: a linear layer followed by batch normalisation equals the layer
+    with folded weights and bias. A dropped epsilon, a swapped mean / variance row or a wrong sign of the shift fails one of the two."""
+    rng = np.random.default_rng(7)
+    channels, features = 12, 20
+    x = rng.standard_normal((30, features)).astype(np.float32)
+    w = rng.standard_normal((channels, features)).astype(np.float32)
+    b = rng.standard_normal(channels).astype(np.float32)
+    gamma = (rng.standard_normal(channels) + 1.5).astype(np.float32)
+    beta = rng.standard_normal(channels).astype(np.float32)
+    stats = np.stack([rng.standard_normal(channels), rng.random(channels) * 1e-3]).astype(np.float32)  # tiny variances: epsilon matters
+    z = O.gemm(x, w, bias=b)
+    normed = O.batchnorm_inference(z, gamma, beta, stats)
+    exact = (z.astype(np.float64) - stats[0]) * gamma / np.sqrt(stats[1].astype(np.float64) + 1e-6) + beta
+    assert np.abs(normed - exact).max() / np.abs(exact).max() <= 1e-6
+    fw, fb = O.fold_batchnorm(w, b, gamma, beta, stats)
+    folded = O.gemm(x, fw, bias=fb)
+    assert np.abs(folded - normed).max() / np.abs(normed).max() <= 1e-5
+    relu = O.batchnorm_inference(z, gamma, beta, stats, act=O.RELU, alpha=0.5, beta=2.0, y=x[:, :channels].copy())
+    assert np.abs(relu - (0.5 * np.maximum(exact, 0.0) + 2.0 * x[:, :channels])).max() / np.abs(exact).max() <= 1e-6
+    none = O.batchnorm_inference(z, None, None, stats)
+    assert np.abs(none - (z.astype(np.float64) - stats[0]) / np.sqrt(stats[1].astype(np.float64) + 1e-6)).max() / np.abs(none).max() <= 1e-6
+    # depthwise weights: channels last
+    dw = rng.standard_normal((3, 3, channels)).astype(np.float32)
+    fdw, _ = O.fold_batchnorm(dw, b, gamma, beta, stats)
+    scale = gamma / np.sqrt(stats[1].astype(np.float64) + 1e-6)
+    assert np.abs(fdw - dw * scale).max() / np.abs(fdw).max() <= 1e-6

@@ -109,3 +109,40 @@ def test_reference_network_bit_exact():
         a = CpuResNet(ps, 2, "oracle").forward(conv(x))
         b = CpuResNet(ps, 2, "reference").forward(conv(x))
         assert mismatches(a, b) == 0
+
+
+@pytest.mark.parametrize("tag", ["f32", "f16"])
+def test_fixtures_heads(golden, tag):
+    g = golden
+    assert mismatches(O.softmax_forward(g["sm_x_" + tag]), g["sm_y_" + tag]) == 0
+    assert mismatches(O.softmax_forward(g["sm3_x_" + tag]), g["sm3_y_" + tag]) == 0
+    assert mismatches(O.global_average_pooling_forward(g["gap_x_" + tag]), g["gap_y_" + tag]) == 0
+    assert mismatches(O.global_average_pooling_forward(g["gap7_x_" + tag]), g["gap7_y_" + tag]) == 0  # scalar kernel only (fp16), 4 + 3 (fp32)
+
+
+def test_fixtures_fold_batchnorm(golden):
+    g = golden
+    for key in ("fd", "fd3"):
+        w, b = O.fold_batchnorm(g[key + "_w"], g[key + "_b"], g[key + "_gamma"], g[key + "_beta"], g[key + "_stats"])
+        assert mismatches(w, g[key + "_w_out"]) == 0 and mismatches(b, g[key + "_b_out"]) == 0
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_reference_heads_bit_exact(dtype):
+    ref = O.reference()
+    rng = np.random.default_rng(2)
+    for shape in ((7, 225), (5, 3), (4, 1), (3, 1000), (2, 64)):
+        x = random_tensor(rng, shape, dtype, 3.0)
+        assert mismatches(O.softmax_forward(x), ref.softmax_forward(x)) == 0
+    for shape in ((3, 13, 14, 136), (2, 15, 15, 256), (1, 1, 1, 8), (2, 5, 6, 7), (2, 3, 3, 37), (1, 4, 4, 3)):
+        x = random_tensor(rng, shape, dtype)
+        assert mismatches(O.global_average_pooling_forward(x), ref.global_average_pooling_forward(x)) == 0
+    if dtype == "float32":
+        for wshape in ((16, 3, 3, 8), (10, 33), (3, 3, 12)):
+            channels = wshape[-1] if len(wshape) == 3 else wshape[0]
+            w, b = random_tensor(rng, wshape, dtype), random_tensor(rng, (channels,), dtype)
+            gamma, beta = random_tensor(rng, (channels,), dtype), random_tensor(rng, (channels,), dtype)
+            stats = np.stack([rng.standard_normal(channels), rng.random(channels) + 0.05]).astype(np.float32)
+            ours, theirs = O.fold_batchnorm(w, b, gamma, beta, stats), ref.fold_batchnorm(w, b, gamma, beta, stats)
+            assert mismatches(ours[0], theirs[0]) == 0 and mismatches(ours[1], theirs[1]) == 0
