@@ -369,13 +369,13 @@ namespace
 	 * (zero outside the image) and runs the input transform. Results are bit-identical to the two separate calls; what is saved is
 	 * the write and re-read of y through HBM (or only the re-read, when y is also needed as a later residual).
 	 */
-	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT>
-	__global__ __launch_bounds__(256, 2) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT, int THREADS>
+	__global__ __launch_bounds__(THREADS, ((VEC <= 2) ? 1024 : 512) / THREADS) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
 			const T *ext, int act, T *__restrict__ next_matrices, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
 	{
 		typedef typename RawVec<T, VEC>::type raw_t;
 		constexpr int CHANNEL_LANES = SLICE / VEC;
-		constexpr int TILE_LANES = 256 / CHANNEL_LANES;
+		constexpr int TILE_LANES = THREADS / CHANNEL_LANES;
 		extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
 		T *image = reinterpret_cast<T*>(lds_bytes); /* [height * width + 1][SLICE]; the extra last pixel stays zero */
 
@@ -402,22 +402,64 @@ namespace
 		else
 			b.zero();
 
-		/* ---- phase 1: output transform into LDS (and to `output`) ---- */
-#pragma clang loop unroll(disable)
-		for (unsigned int in_image = tile_lane; in_image < tiles_per_image; in_image += TILE_LANES)
+		/*
+		 * The residual slice of this image goes straight into the image buffer with direct-to-LDS loads (16 bytes per lane, no staging
+		 * registers): phase 1 then adds it from LDS and overwrites it in place with y. Every (pixel, channel) of the buffer is read and
+		 * written by the one thread that owns its tile, so no further synchronisation is needed inside phase 1.
+		 */
+		if constexpr (HAS_EXT)
 		{
-			const unsigned int tile_idx = batch * tiles_per_image + in_image;
-			const int tile_x = in_image / tiles_w;
-			const int x0 = 4 * tile_x;
-			const int y0 = 4 * (in_image - tile_x * tiles_w);
+			typedef __attribute__((address_space(3))) void *lds_ptr_t;
+			typedef __attribute__((address_space(1))) const void *global_ptr_t;
+			constexpr int CHUNKS_PER_PIXEL = SLICE * static_cast<int>(sizeof(T)) / 16;
+			const int total_chunks = zero_pixel * CHUNKS_PER_PIXEL;
+			const uint8_t *ext_slice = reinterpret_cast<const uint8_t*>(ext + static_cast<size_t>(batch) * zero_pixel * channels + slice * SLICE);
+			const int lane = threadIdx.x & 63;
+			for (int base = (threadIdx.x >> 6) * 64; base < total_chunks; base += THREADS)
+			{
+				const int chunk = base + lane;
+				if (chunk < total_chunks)
+				{
+					const int px = chunk / CHUNKS_PER_PIXEL;
+					const int part = chunk - px * CHUNKS_PER_PIXEL;
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (ext_slice + static_cast<size_t>(px) * channels * sizeof(T) + part * 16),
+							(lds_ptr_t) (lds_bytes + base * 16), 16, 0, 0);
+				}
+			}
+		}
 
-			const T *src = matrices + static_cast<size_t>(tile_idx) * channels + channel;
-			raw_t raw[6][6];
+		/* ---- phase 1: output transform into LDS (and to `output`) ---- */
+		const unsigned int image_base = batch * height * width;
+		raw_t raw[6][6];
+		auto load_matrices = [&](unsigned int in_image) __attribute__((always_inline))
+		{
+			const T *src = matrices + static_cast<size_t>(batch * tiles_per_image + in_image) * channels + channel;
 #pragma unroll
 			for (int row = 0; row < 6; row++)
 #pragma unroll
 				for (int col = 0; col < 6; col++)
 					raw[row][col] = *reinterpret_cast<const raw_t*>(src + static_cast<size_t>(row * 6 + col) * matrix_stride);
+		};
+		unsigned int in_image = tile_lane;
+		bool loaded = false;
+		if constexpr (HAS_EXT)
+		{ /* the first tile's matrices are requested before the wait, so that they fly together with the residual slice */
+			if (in_image < tiles_per_image)
+			{
+				load_matrices(in_image);
+				loaded = true;
+			}
+			__syncthreads(); /* waits for this wavefront's loads, then for everyone's: the residual slice is complete */
+		}
+#pragma clang loop unroll(disable)
+		while (in_image < tiles_per_image)
+		{
+			if (!loaded)
+				load_matrices(in_image);
+			loaded = false;
+			const int tile_x = in_image / tiles_w;
+			const int x0 = 4 * tile_x;
+			const int y0 = 4 * (in_image - tile_x * tiles_w);
 
 			int pixel[4][4]; /* pixel index within the image, clamped */
 #pragma unroll
@@ -425,16 +467,6 @@ namespace
 #pragma unroll
 				for (int col = 0; col < 4; col++)
 					pixel[row][col] = min(x0 + row, height - 1) * width + min(y0 + col, width - 1);
-			const unsigned int image_base = batch * height * width;
-			raw_t residual[4][4];
-			if constexpr (HAS_EXT)
-			{
-#pragma unroll
-				for (int row = 0; row < 4; row++)
-#pragma unroll
-					for (int col = 0; col < 4; col++)
-						residual[row][col] = *reinterpret_cast<const raw_t*>(ext + (image_base + pixel[row][col]) * channels + channel);
-			}
 
 			float tmp[4][6][VEC];
 #pragma unroll
@@ -462,13 +494,17 @@ namespace
 #pragma unroll
 				for (int col = 0; col < 4; col++)
 				{
+					T *in_lds = image + pixel[row][col] * SLICE + channel_local;
+					raw_t residual;
+					if constexpr (HAS_EXT)
+						residual = *reinterpret_cast<const raw_t*>(in_lds);
 					Vec<T, VEC> out;
 #pragma unroll
 					for (int c = 0; c < VEC; c++)
 					{
 						float t = res[col][c] + b.v[c];
 						if constexpr (HAS_EXT)
-							t = t + RawVec<T, VEC>::get(residual[row][col], c);
+							t = t + RawVec<T, VEC>::get(residual, c);
 						if constexpr (ACT == 1)
 							t = fmaxf(t, 0.0f);
 						if constexpr (ACT == 2)
@@ -481,12 +517,13 @@ namespace
 					}
 					if ((x0 + row) < height && (y0 + col) < width)
 					{
-						out.store(image + pixel[row][col] * SLICE + channel_local);
+						out.store(in_lds);
 						if (output != nullptr)
 							out.store(output + (image_base + pixel[row][col]) * channels + channel);
 					}
 				}
 			}
+			in_image += TILE_LANES;
 		}
 		__syncthreads();
 
@@ -679,16 +716,15 @@ namespace
 		MLHIP_CHECK(hipGetLastError());
 	}
 	/* fused output + next input transform: channels must be a multiple of 64 and 4-element accesses aligned */
-	template<typename T, int SLICE>
+	template<typename T, int SLICE, int VEC, int THREADS>
 	void launch_output_input(hipStream_t stream, const mlTensor_t &matrices, const mlTensor_t &bias, const mlTensor_t &ext, const mlShape_t &shape, void *output,
 			mlActivationType_t act, mlTensor_t &next)
 	{
-		constexpr int VEC = 4;
 		const int batch = shape.dim[0], height = shape.dim[1], width = shape.dim[2], channels = shape.dim[3];
 		const int tiles_h = ceil_div(height, 4), tiles_w = ceil_div(width, 4);
 		const size_t lds = static_cast<size_t>(height * width + 1) * SLICE * sizeof(T);
 		MLHIP_REQUIRE(lds <= 160 * 1024, "Winograd fused transform: image too large for LDS");
-		const dim3 grid(static_cast<unsigned int>(batch) * (channels / SLICE)), block(256);
+		const dim3 grid(static_cast<unsigned int>(batch) * (channels / SLICE)), block(THREADS);
 		const T *in = ptr<const T>(matrices);
 		T *out = reinterpret_cast<T*>(output);
 		const T *b = ptr<const T>(bias);
@@ -698,7 +734,7 @@ namespace
 		const int mode = (act == ACTIVATION_LINEAR) ? 0 : ((act == ACTIVATION_RELU) ? 1 : 2);
 #define MLHIP_LAUNCH_FUSED(MODE, EXT) \
 		do { \
-			auto kernel = kernel_output_input_transform_4x4_3x3<T, VEC, SLICE, MODE, EXT>; \
+			auto kernel = kernel_output_input_transform_4x4_3x3<T, VEC, SLICE, MODE, EXT, THREADS>; \
 			if (lds > 64 * 1024) \
 				ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), static_cast<int>(lds)); \
 			hipLaunchKernelGGL(kernel, grid, block, lds, stream, in, out, b, e, a, nxt, batch, height, width, channels, tiles_h, tiles_w); \
@@ -825,22 +861,12 @@ extern "C"
 			return;
 		}
 		mlTensor_t next = next_matrices;
-		/* wider channel slices make longer contiguous segments in memory, as long as two workgroups still fit the LDS of a CU */
-		const bool wide = false && (channels % 128 == 0) && static_cast<size_t>(output_shape.dim[1] * output_shape.dim[2] + 1) * 128 * esize <= 80 * 1024;
+		/* 64-channel slices, 256 threads, two workgroups per CU. Measured alternatives that were not faster: slices of 128 or 256 channels
+		 * (longer contiguous segments) with 512 or 1024 threads, and 2-element vectors at twice the occupancy. */
 		if (matrices.dtype == DTYPE_FLOAT16)
-		{
-			if (wide)
-				launch_output_input<half_t, 128>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
-			else
-				launch_output_input<half_t, 64>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
-		}
+			launch_output_input<half_t, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
 		else
-		{
-			if (wide)
-				launch_output_input<float, 128>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
-			else
-				launch_output_input<float, 64>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
-		}
+			launch_output_input<float, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
 	}
 } /* extern "C" */
 

@@ -48,6 +48,7 @@ class ResNet:
         """params_host: list from make_parameters; to_storage: fp32 ndarray -> ndarray in the storage type (identity or fp16 bits)."""
         self.context = context
         self.fused = fused
+        self.fuse_block_boundary = True  # False: fuse only inside the residual blocks (for measurements)
         self.dtype = ml.dtype_of(dtype)
         self.batch, self.board, self.channels, self.blocks = batch, board, channels, blocks
         self.chunk = min(chunk or batch, batch)
@@ -122,12 +123,14 @@ class ResNet:
                 conv1.winograd_output_into(conv2, n, None if self.channels % 64 == 0 else b, None, ws)  # only conv2 reads this result
                 ml.set_timer_label("block_conv2")
                 conv2.winograd_gemm(n, ws)
-                # with a residual to read and the block output to write the fused launch is not faster than the two transforms
-                # (measured: its register footprint halves the occupancy), so the block boundary stays unfused
-                conv2.winograd_output(c, a, ws)  # c = next block's input and residual
-                if blk + 1 < self.blocks:
-                    ml.set_timer_label("block_conv1")
-                    L[3 + 2 * blk].winograd_input(c, ws)
+                # c = next block's input and residual: written to memory and, inside the same launch, transformed for the next block
+                if blk + 1 < self.blocks and self.channels % 64 == 0 and self.fuse_block_boundary:
+                    conv2.winograd_output_into(L[3 + 2 * blk], n, c, a, ws)
+                else:
+                    conv2.winograd_output(c, a, ws)
+                    if blk + 1 < self.blocks:
+                        ml.set_timer_label("block_conv1")
+                        L[3 + 2 * blk].winograd_input(c, ws)
                 a, c = c, a
             ml.set_timer_label("head")
             L[-1].forward([a], self._view_batch(self.output, start, n), ws)
