@@ -98,6 +98,7 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--unfused", action="store_true", help="run every layer as the reference's three calls (no cross-layer transform fusion)")
+    ap.add_argument("--layer-launch", action="store_true", help="experimental: product and both transforms of a layer as one launch (slower)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one 256 MiB copy kernel (kernel_axpy3) for scaling hardware counters")
     args = ap.parse_args()
@@ -120,6 +121,7 @@ def main():
     if args.copy_calibration:
         copy_calibration(ml, ctx)
     net = ResNet(ctx, batch, board, planes, channels, blocks, dtype, params, to_storage, chunk=chunk, fused=not args.unfused)
+    net.fuse_layers = bool(args.layer_launch) and not args.unfused
     net.setInput(to_storage(x))
 
     for _ in range(args.warmup):

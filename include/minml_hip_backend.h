@@ -116,6 +116,22 @@ extern "C"
 	void hip_winograd_output_input_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
 			mlShape_t output_shape, void *output, mlActivationType_t act, mlTensor_t next_matrices);
 
+	/*
+	 * hip_winograd_layer_forward: one whole 3x3 layer between two sets of Winograd matrices, in one launch:
+	 *   input_matrices [36, tiles, Cin] x weight_matrices [36, Cout, Cin]^T -> output transform (+ bias, + ext, act) -> y (`output`, may be
+	 *   NULL) -> input transform -> next_matrices [36, tiles, Cout]
+	 * i.e. hip_gemm_batched followed by hip_winograd_output_input_transform, with identical results. For fp16, 256 -> 256 channels,
+	 * boards of 16 tiles (13x13 .. 16x16), batches that are multiples of 4 (at least 32) and linear / ReLU activation the product never
+	 * leaves the L2 cache; every other case runs the two calls through `output_matrices` [36, tiles, Cout], which must then be given.
+	 * No counterpart in the reference (src/layers/Conv2D.cpp:365-378 calls the three steps one by one).
+	 * hip_winograd_layer_errors waits for the context's stream and returns how many workgroups of such launches gave up waiting for
+	 * one another since the last call (0 unless the device was shared with other work; results are then invalid).
+	 */
+	void hip_winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
+			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
+			mlTensor_t next_matrices);
+	int hip_winograd_layer_errors(mlContext_t context);
+
 	/* ---- GEMMs (reference: cuda_backend.h:147-154; semantics of src/backend/cpu/gemm/gemm.cpp:34-83).
 	 *      C.dtype == INT32 selects the int8 x int8 -> int32 product (src/backend/cuda/gemms.cpp:119-130). ---- */
 	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C);

@@ -83,6 +83,8 @@ SIGNATURES = {
     "winograd_input_transform": (None, [_vp, _i, _T, _T]),
     "winograd_output_transform": (None, [_vp, _i, _T, _T, _T, _T, _i]),
     "winograd_output_input_transform": (None, [_vp, _i, _T, _T, _T, _S, _vp, _i, _T]),
+    "winograd_layer_forward": (None, [_vp, _i, _T, _T, _T, _T, _T, _S, _vp, _i, _T]),
+    "winograd_layer_errors": (_i, [_vp]),
     "gemm_v2": (None, [_vp, _c, _c, _f, _T, _T, _f, _T]),
     "gemm_batched_v2": (None, [_vp, _c, _c, _f, _T, _T, _f, _T]),
     "gemm": (None, [_vp, _i, _S, _vp, _S, _vp, _S, _vp, _c, _c, _f, _f]),

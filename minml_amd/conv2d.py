@@ -159,6 +159,22 @@ class Conv2D:
         out_shape = (batch,) + self.output_shape[1:]
         ml.winogradOutputInputTransform(self.context, self.weight_shape, output_matrices, out_shape, output, self.bias, add, self.activation, next_input)
 
+    def winograd_layer_into(self, next_layer, batch, output, add, workspace):
+        """Product, output transform and `next_layer`'s input transform in one call, from this layer's input matrices already in the
+        workspace. The next layer's input matrices replace this layer's at element 0: a tile's rows are rewritten only after every
+        position of that tile has been multiplied."""
+        ctx = self.context
+        if self.transformed_weights is None:
+            self.transformed_weights = ml.Tensor(get_weight_matrices_shape(self.weight_shape, self.winograd_tile_size), self.dtype, ctx.device_index)
+            ml.winogradWeightTransform(ctx, self.weights, self.transformed_weights, False)
+        input_matrices, output_matrices = self._winograd_views(batch, workspace)
+        next_input, _ = next_layer._winograd_views(batch, workspace)
+        if next_input.volume() > input_matrices.volume():
+            raise ValueError("the next layer's input matrices would overlap this layer's output matrices in the workspace")
+        out_shape = (batch,) + self.output_shape[1:]
+        ml.winogradLayerForward(ctx, self.weight_shape, input_matrices, self.transformed_weights, output_matrices, out_shape, output, self.bias, add,
+                                self.activation, next_input)
+
     def _forward_int8(self, x, add, output, workspace):
         ctx = self.context
         ext_transform = self.input_transforms[1] if add is not None else (1.0, 0.0)

@@ -334,6 +334,30 @@ def winogradOutputInputTransform(context, weight_shape, matrices, output_shape, 
             act_of(act), next_matrices.desc())
 
 
+def winogradLayerForward(context, weight_shape, input_matrices, weight_matrices, output_matrices, output_shape, output, bias, add, act, next_matrices):
+    """Batched product, output transform and the next 3x3 layer's input transform in one call (no counterpart in the reference's
+    math.hpp): identical to gemmBatched into `output_matrices` followed by winogradOutputInputTransform. For fp16, 256 channels and 16
+    tiles per image the product stays in the L2 cache and `output_matrices` is not touched."""
+    tile = get_winograd_tile(weight_shape, input_matrices.shape)
+    _require_winograd_supported(tile, weight_shape[1], input_matrices.dtype)
+    _require(_same_dtype(input_matrices, weight_matrices, output_matrices, next_matrices, output, bias, add), "dtype mismatch")
+    b, h, w, c = output_shape
+    tiles = b * ((h + 3) // 4) * ((w + 3) // 4)
+    _require(input_matrices.shape == (36, tiles, weight_shape[3]) and weight_matrices.shape == (36, c, weight_shape[3]), "input / weight matrices shape")
+    _require(output_matrices.shape == (36, tiles, c) and next_matrices.shape == (36, tiles, c), "output / next matrices must be [36, tiles, C]")
+    _require(output is None or output.shape == tuple(output_shape), "output must have the given shape")
+    _require(bias is None or bias.isEmpty() or bias.volume() == c, "bias must be [C]")
+    _require(add is None or add.isEmpty() or add.shape == tuple(output_shape), "add must have the output's shape")
+    _require(output is not None or c % 64 == 0, "without an output tensor the channel count must be a multiple of 64")
+    _launch("winograd_layer_forward", context.handle, tile, input_matrices.desc(), weight_matrices.desc(), output_matrices.desc(), _desc(bias), _desc(add),
+            B.make_shape(output_shape), _ptr(output), act_of(act), next_matrices.desc())
+
+
+def winogradLayerErrors(context):
+    """Waits for the context and returns how many workgroups of whole-layer launches gave up waiting since the last call (0 = all good)."""
+    return int(B.fn("winograd_layer_errors")(context.handle))
+
+
 def _gemm_dims(opA, A, opB, Bm):
     ta, tb = opA in "tT", opB in "tT"
     _require(opA in "ntNT" and opB in "ntNT", "op must be n or t")

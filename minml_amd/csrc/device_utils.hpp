@@ -127,6 +127,28 @@ namespace mlhip
 					*reinterpret_cast<vt*>(p) = tmp;
 				}
 			}
+			/* the same store marked non-temporal: the line is not meant to be kept in the caches */
+			__device__ __forceinline__ void store_streaming(T *p) const
+			{
+				if constexpr (sizeof(T) == 4)
+				{
+					typedef float vt __attribute__((ext_vector_type(N)));
+					vt tmp;
+#pragma unroll
+					for (int i = 0; i < N; i++)
+						tmp[i] = v[i];
+					__builtin_nontemporal_store(tmp, reinterpret_cast<vt*>(p));
+				}
+				else
+				{
+					typedef uint32_t vt __attribute__((ext_vector_type(N / 2)));
+					vt tmp;
+#pragma unroll
+					for (int i = 0; i < N / 2; i++)
+						tmp[i] = pack_rtz(v[2 * i], v[2 * i + 1]);
+					__builtin_nontemporal_store(tmp, reinterpret_cast<vt*>(p));
+				}
+			}
 			__device__ __forceinline__ void zero()
 			{
 #pragma unroll

@@ -17,6 +17,10 @@
  */
 #include "common.hpp"
 #include "device_utils.hpp"
+#include "gemm_stream.hpp"
+
+#include <map>
+#include <mutex>
 
 #pragma clang fp contract(off)
 
@@ -360,34 +364,36 @@ namespace
 		}
 	}
 
-	/*
-	 * Output transform of one layer fused with the input transform of the next 3x3 layer:
-	 *   matrices [36][tiles][C] (+ bias, + ext) -> y [B][H][W][C] (written only if `output` is given) -> next_matrices [36][tiles][C]
-	 * One workgroup owns one image and a slice of SLICE channels: its 256 threads are 256 / (SLICE / VEC) tile lanes x SLICE / VEC
-	 * channel lanes. Phase 1 runs the output transform of the image's tiles (same arithmetic and epilogue as the stand-alone kernel) and
-	 * leaves y, rounded to the storage type as the stand-alone kernel would store it, in LDS; phase 2 reads the 6x6 windows back
-	 * (zero outside the image) and runs the input transform. Results are bit-identical to the two separate calls; what is saved is
-	 * the write and re-read of y through HBM (or only the re-read, when y is also needed as a later residual).
-	 */
-	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT, int THREADS>
-	__global__ __launch_bounds__(THREADS, ((VEC <= 2) ? 1024 : 512) / THREADS) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
-			const T *ext, int act, T *__restrict__ next_matrices, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
+	/* one image's share of a fused output -> input transform: where its matrices, pixels and next matrices lie */
+	template<typename T>
+	struct FusedImage
+	{
+			const T *matrices; /* position 0, first tile of the image, channel 0 */
+			size_t matrix_stride; /* elements between two positions */
+			T *output; /* first pixel of the image, channel 0; nullptr: y is not written */
+			const T *ext; /* first pixel of the image's residual (only read when HAS_EXT) */
+			const T *bias; /* [channels] or nullptr */
+			T *next_matrices; /* like `matrices`, for the next layer */
+			size_t next_stride;
+			int act, height, width, channels, tiles_h, tiles_w;
+			int slice; /* which SLICE channels of the image this workgroup owns */
+	};
+
+	/* phase 1: output transform of the image's tiles into the LDS image [height * width + 1][SLICE] (and to g.output) */
+	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT, int THREADS, bool STREAM = false>
+	__device__ __forceinline__ void fused_transform_phase1(const FusedImage<T> &g, uint8_t *lds_bytes)
 	{
 		typedef typename RawVec<T, VEC>::type raw_t;
 		constexpr int CHANNEL_LANES = SLICE / VEC;
 		constexpr int TILE_LANES = THREADS / CHANNEL_LANES;
-		extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
-		T *image = reinterpret_cast<T*>(lds_bytes); /* [height * width + 1][SLICE]; the extra last pixel stays zero */
-
-		const unsigned int slices = channels / SLICE;
-		const unsigned int batch = blockIdx.x / slices;
-		const unsigned int slice = blockIdx.x - batch * slices;
+		T *image = reinterpret_cast<T*>(lds_bytes); /* the extra last pixel stays zero */
+		const int height = g.height, width = g.width, channels = g.channels;
 		const int channel_local = (threadIdx.x % CHANNEL_LANES) * VEC;
-		const unsigned int channel = slice * SLICE + channel_local;
+		const unsigned int channel = g.slice * SLICE + channel_local;
 		const int tile_lane = threadIdx.x / CHANNEL_LANES;
-		const unsigned int tiles_per_image = tiles_h * tiles_w;
-		const unsigned int nb_of_tiles = batch_size * tiles_per_image;
-		const size_t matrix_stride = static_cast<size_t>(nb_of_tiles) * channels;
+		const unsigned int tiles_per_image = g.tiles_h * g.tiles_w;
+		const int tiles_w = g.tiles_w;
+		const size_t matrix_stride = g.matrix_stride;
 		const int zero_pixel = height * width;
 
 		if (tile_lane == 0)
@@ -397,8 +403,8 @@ namespace
 			z.store(image + zero_pixel * SLICE + channel_local);
 		}
 		Vec<T, VEC> b;
-		if (bias != nullptr)
-			b.load(bias + channel);
+		if (g.bias != nullptr)
+			b.load(g.bias + channel);
 		else
 			b.zero();
 
@@ -413,7 +419,7 @@ namespace
 			typedef __attribute__((address_space(1))) const void *global_ptr_t;
 			constexpr int CHUNKS_PER_PIXEL = SLICE * static_cast<int>(sizeof(T)) / 16;
 			const int total_chunks = zero_pixel * CHUNKS_PER_PIXEL;
-			const uint8_t *ext_slice = reinterpret_cast<const uint8_t*>(ext + static_cast<size_t>(batch) * zero_pixel * channels + slice * SLICE);
+			const uint8_t *ext_slice = reinterpret_cast<const uint8_t*>(g.ext + g.slice * SLICE);
 			const int lane = threadIdx.x & 63;
 			for (int base = (threadIdx.x >> 6) * 64; base < total_chunks; base += THREADS)
 			{
@@ -423,17 +429,15 @@ namespace
 					const int px = chunk / CHUNKS_PER_PIXEL;
 					const int part = chunk - px * CHUNKS_PER_PIXEL;
 					__builtin_amdgcn_global_load_lds((global_ptr_t) (ext_slice + static_cast<size_t>(px) * channels * sizeof(T) + part * 16),
-							(lds_ptr_t) (lds_bytes + base * 16), 16, 0, 0);
+							(lds_ptr_t) (lds_bytes + base * 16), 16, 0, STREAM ? 2 : 0);
 				}
 			}
 		}
 
-		/* ---- phase 1: output transform into LDS (and to `output`) ---- */
-		const unsigned int image_base = batch * height * width;
 		raw_t raw[6][6];
 		auto load_matrices = [&](unsigned int in_image) __attribute__((always_inline))
 		{
-			const T *src = matrices + static_cast<size_t>(batch * tiles_per_image + in_image) * channels + channel;
+			const T *src = g.matrices + static_cast<size_t>(in_image) * channels + channel;
 #pragma unroll
 			for (int row = 0; row < 6; row++)
 #pragma unroll
@@ -508,30 +512,49 @@ namespace
 						if constexpr (ACT == 1)
 							t = fmaxf(t, 0.0f);
 						if constexpr (ACT == 2)
-						{
+						{ /* the reference stores y and then runs the activation over it: round through the storage type in between */
 							if constexpr (sizeof(T) == 2)
 								t = half_bits_to_float(half_bits_rtz(t));
-							t = activate(act, t);
+							t = activate(g.act, t);
 						}
 						out.v[c] = t;
 					}
 					if ((x0 + row) < height && (y0 + col) < width)
 					{
 						out.store(in_lds);
-						if (output != nullptr)
-							out.store(output + (image_base + pixel[row][col]) * channels + channel);
+						if (g.output != nullptr)
+						{
+							if constexpr (STREAM)
+								out.store_streaming(g.output + static_cast<size_t>(pixel[row][col]) * channels + channel);
+							else
+								out.store(g.output + static_cast<size_t>(pixel[row][col]) * channels + channel);
+						}
 					}
 				}
 			}
 			in_image += TILE_LANES;
 		}
-		__syncthreads();
+	}
 
-		/* ---- phase 2: input transform of the next layer out of LDS ---- */
+	/* phase 2: input transform of the next layer out of the LDS image (all of phase 1 must have finished: barrier in between) */
+	template<typename T, int VEC, int SLICE, int THREADS, bool STREAM = false>
+	__device__ __forceinline__ void fused_transform_phase2(const FusedImage<T> &g, const uint8_t *lds_bytes)
+	{
+		typedef typename RawVec<T, VEC>::type raw_t;
+		constexpr int CHANNEL_LANES = SLICE / VEC;
+		constexpr int TILE_LANES = THREADS / CHANNEL_LANES;
+		const T *image = reinterpret_cast<const T*>(lds_bytes);
+		const int height = g.height, width = g.width, channels = g.channels;
+		const int channel_local = (threadIdx.x % CHANNEL_LANES) * VEC;
+		const unsigned int channel = g.slice * SLICE + channel_local;
+		const int tile_lane = threadIdx.x / CHANNEL_LANES;
+		const unsigned int tiles_per_image = g.tiles_h * g.tiles_w;
+		const int tiles_w = g.tiles_w;
+		const size_t next_stride = g.next_stride;
+		const int zero_pixel = height * width;
 #pragma clang loop unroll(disable)
 		for (unsigned int in_image = tile_lane; in_image < tiles_per_image; in_image += TILE_LANES)
 		{
-			const unsigned int tile_idx = batch * tiles_per_image + in_image;
 			const int tile_x = in_image / tiles_w;
 			const int x0 = 4 * tile_x - 1;
 			const int y0 = 4 * (in_image - tile_x * tiles_w) - 1;
@@ -573,7 +596,7 @@ namespace
 					for (int c = 0; c < VEC; c++)
 						tmp[row][col][c] = res[row][c];
 			}
-			T *dst = next_matrices + static_cast<size_t>(tile_idx) * channels + channel;
+			T *dst = g.next_matrices + static_cast<size_t>(in_image) * channels + channel;
 #pragma unroll
 			for (int row = 0; row < 6; row++)
 			{
@@ -586,8 +609,290 @@ namespace
 #pragma unroll
 					for (int c = 0; c < VEC; c++)
 						out.v[c] = res[col][c];
-					out.store(dst + static_cast<size_t>(row * 6 + col) * matrix_stride);
+					if constexpr (STREAM)
+						out.store_streaming(dst + static_cast<size_t>(row * 6 + col) * next_stride);
+					else
+						out.store(dst + static_cast<size_t>(row * 6 + col) * next_stride);
 				}
+			}
+		}
+	}
+
+	/*
+	 * Output transform of one layer fused with the input transform of the next 3x3 layer:
+	 *   matrices [36][tiles][C] (+ bias, + ext) -> y [B][H][W][C] (written only if `output` is given) -> next_matrices [36][tiles][C]
+	 * One workgroup owns one image and a slice of SLICE channels: its THREADS threads are THREADS / (SLICE / VEC) tile lanes x
+	 * SLICE / VEC channel lanes. Phase 1 runs the output transform of the image's tiles (same arithmetic and epilogue as the stand-alone
+	 * kernel) and leaves y, rounded to the storage type as the stand-alone kernel would store it, in LDS; phase 2 reads the 6x6 windows
+	 * back (zero outside the image) and runs the input transform. Results are bit-identical to the two separate calls; what is saved is
+	 * the write and re-read of y through HBM (or only the re-read, when y is also needed as a later residual).
+	 */
+	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT, int THREADS>
+	__global__ __launch_bounds__(THREADS, ((VEC <= 2) ? 1024 : 512) / THREADS) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+			const T *ext, int act, T *__restrict__ next_matrices, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
+	{
+		extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
+		const unsigned int slices = channels / SLICE;
+		const unsigned int batch = blockIdx.x / slices;
+		const unsigned int tiles_per_image = tiles_h * tiles_w;
+		const size_t image_pixels = static_cast<size_t>(batch) * height * width;
+		FusedImage<T> g;
+		g.matrix_stride = static_cast<size_t>(batch_size) * tiles_per_image * channels;
+		g.next_stride = g.matrix_stride;
+		g.matrices = matrices + static_cast<size_t>(batch) * tiles_per_image * channels;
+		g.next_matrices = next_matrices + static_cast<size_t>(batch) * tiles_per_image * channels;
+		g.output = (output != nullptr) ? output + image_pixels * channels : nullptr;
+		g.ext = HAS_EXT ? ext + image_pixels * channels : nullptr;
+		g.bias = bias;
+		g.act = act;
+		g.height = height;
+		g.width = width;
+		g.channels = channels;
+		g.tiles_h = tiles_h;
+		g.tiles_w = tiles_w;
+		g.slice = blockIdx.x - batch * slices;
+		fused_transform_phase1<T, VEC, SLICE, ACT, HAS_EXT, THREADS>(g, lds_bytes);
+		__syncthreads();
+		fused_transform_phase2<T, VEC, SLICE, THREADS>(g, lds_bytes);
+	}
+
+	/* ---------------------------------------------------------------------------------------------------------------------
+	 * A whole 3x3 layer in one launch (fp16, 256 -> 256 channels, 16 tiles per image):
+	 *   V [36][T][256] x U [36][256][256]^T -> M -> output transform (+ bias, + ext, activation) -> y -> input transform -> V' [36][T][256]
+	 * The product M never reaches HBM: it lives in the L2 of one XCD between the workgroups that make it and those that transform it.
+	 *
+	 * 512 workgroups of 256 threads, all resident at once (two per CU), find out which XCD they run on and take a role there:
+	 *   36 GEMM workgroups, one per matrix position: the position's B operand (256 x 256) stays in registers for the whole launch
+	 *     (4 wavefronts x 64 columns); for every chunk of 64 tiles (4 images) the XCD owns, 32 KB of A come HBM -> LDS by direct-to-LDS
+	 *     loads (requested one chunk ahead), 64 MFMAs per wavefront make the 64 x 256 product, and it is stored to a scratch buffer
+	 *     that is reused every LAYER_BUFFERS chunks and therefore stays in the XCD's L2;
+	 *   28 transform workgroups: each takes (image, 64-channel slice) tasks of a finished chunk in turn and runs the fused
+	 *     output -> input transform on them, reading M from the scratch buffer.
+	 * Two counters per chunk order them: `produced` (36 arrivals: the chunk's M is complete) and `consumed` (16 arrivals: every task
+	 * has read its part, the buffer may be overwritten). Stores are acknowledged by the L2 before a workgroup arrives, and a consumer
+	 * drops its L1 lines after the wait, so data passes between CUs of one XCD without any L2 write-back. Every wait is bounded: a
+	 * workgroup that gives up counts itself in the error word and leaves, and the others follow, so the grid always drains.
+	 * Streaming traffic (A, the residual, y and V') is marked non-temporal so that it evicts as little of M as possible.
+	 *
+	 * Status (MI355X, batch 1024): results are bit-identical to the separate launches, but the launch takes about 430 us where the
+	 * streaming product plus the fused transform take about 290 us. Measured reasons: only 28 of the 64 workgroups of an XCD transform,
+	 * and a task is a chain of latencies (about 14 us), so the transform side limits the pipeline; while a chunk of M waits for it, two
+	 * chunks' worth of streaming data pass through the 4 MiB L2 and evict about 80 % of M to HBM after all (HBM writes 548 MB per
+	 * launch where 302 MB are V'). A probe of the mechanism alone shows what is available: data ping-ponged between CUs of one XCD stays
+	 * out of HBM (22 MB written for 3.4 GB exchanged), an XCD-wide barrier costs about 0.8 us, dropping the L1 costs little, whereas an
+	 * agent-scope acquire fence costs about 8 us.
+	 * ------------------------------------------------------------------------------------------------------------------- */
+	constexpr int LAYER_CHUNK_TILES = 64; /* rows of one GEMM unit = 4 images of 16 tiles */
+	constexpr int LAYER_CHANNELS = 256;
+	constexpr int LAYER_BUFFERS = 2; /* scratch copies of a chunk's M per XCD: 2 x 36 x 64 x 256 x 2 bytes = 2.25 MiB of the 4 MiB L2 */
+	constexpr int LAYER_GEMM_WORKGROUPS = 36, LAYER_WORKGROUPS_PER_XCD = 64, LAYER_XCDS = 8;
+	constexpr int LAYER_TRANSFORM_WORKGROUPS = LAYER_WORKGROUPS_PER_XCD - LAYER_GEMM_WORKGROUPS;
+	constexpr int LAYER_TASKS_PER_CHUNK = 16; /* 4 images x 4 slices of 64 channels */
+	constexpr int LAYER_MAX_CHUNKS = 128; /* chunks per XCD that the counters cover: batch <= 8 * 128 * 4 images */
+	constexpr size_t LAYER_CHUNK_ELEMENTS = static_cast<size_t>(36) * LAYER_CHUNK_TILES * LAYER_CHANNELS;
+
+	struct LayerSync /* one per XCD; every counter on a cache line of its own */
+	{
+			unsigned int ticket, pad0[15];
+			unsigned int produced[LAYER_MAX_CHUNKS][16];
+			unsigned int consumed[LAYER_MAX_CHUNKS][16];
+	};
+
+	__device__ __forceinline__ int xcc_id()
+	{
+		return __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 7; /* hardware register XCC_ID, bits 3:0 */
+	}
+	/* polls until *counter >= target; false after `limit` polls */
+	__device__ __forceinline__ bool wait_for_counter(unsigned int *counter, unsigned int target, unsigned int limit)
+	{
+		unsigned int polls = 0;
+		while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target)
+		{
+			if (++polls >= limit)
+				return false;
+			__builtin_amdgcn_s_sleep(1);
+		}
+		return true;
+	}
+
+	template<int ACT, bool HAS_EXT>
+	__global__ __launch_bounds__(256, 2) void kernel_winograd_layer_f16(const half_t *V, const half_t *U, const half_t *bias, const half_t *ext, half_t *output,
+			half_t *next_matrices, half_t *scratch, LayerSync *sync, unsigned int *errors, int batch, int height, int width, int tiles_h, int tiles_w,
+			int act, unsigned int spin_limit)
+	{
+		typedef MfmaTraits<half_t> Traits;
+		typedef Traits::acc_vec acc_vec;
+		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+		__shared__ unsigned int s_word;
+		const int xcd = xcc_id();
+		LayerSync &my = sync[xcd];
+		if (threadIdx.x == 0)
+			s_word = __hip_atomic_fetch_add(&my.ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+		__syncthreads();
+		const unsigned int role = s_word;
+		__syncthreads();
+		if (role >= LAYER_WORKGROUPS_PER_XCD)
+			return; /* more workgroups on this XCD than roles */
+
+		const int total_chunks = batch / 4;
+		const int my_chunks = (total_chunks - xcd + LAYER_XCDS - 1) / LAYER_XCDS; /* chunks xcd, xcd + 8, ... */
+		half_t *my_scratch = scratch + static_cast<size_t>(xcd) * LAYER_BUFFERS * LAYER_CHUNK_ELEMENTS;
+		const size_t all_tiles = static_cast<size_t>(batch) * 16;
+		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+		if (role < LAYER_GEMM_WORKGROUPS)
+		{
+			const int p = role;
+			const int frag_row = lane & 31, half_sel = lane >> 5;
+			uint4_t b_regs[2][16]; /* 2 groups of 32 columns x 16 k steps */
+			{
+				const uint8_t *b_base = reinterpret_cast<const uint8_t*>(U + static_cast<size_t>(p) * LAYER_CHANNELS * LAYER_CHANNELS);
+#pragma unroll
+				for (int cg = 0; cg < 2; cg++)
+				{
+					const uint8_t *row = b_base + static_cast<size_t>(wave * 64 + cg * 32 + frag_row) * 512 + half_sel * 16;
+#pragma unroll
+					for (int k = 0; k < 16; k++)
+						b_regs[cg][k] = *reinterpret_cast<const uint4_t*>(row + k * 32);
+				}
+			}
+			/* a chunk of A: 64 rows x 512 bytes, kept as 4 k stages of 64 rows x 128 bytes; a wavefront moves 8 blocks of 1 KB */
+			int source_offset[8];
+#pragma unroll
+			for (int i = 0; i < 8; i++)
+			{
+				const int block = wave + 4 * i;
+				const int row = (block & 7) * 8 + (lane >> 3);
+				source_offset[i] = row * 512 + (block >> 3) * 128 + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+			}
+			const uint8_t *a_base = reinterpret_cast<const uint8_t*>(V + static_cast<size_t>(p) * all_tiles * LAYER_CHANNELS);
+			auto request_chunk = [&](int ci) __attribute__((always_inline))
+			{
+				const uint8_t *a = a_base + static_cast<size_t>(xcd + LAYER_XCDS * ci) * LAYER_CHUNK_TILES * 512;
+				uint8_t *slot = lds + (ci & 1) * 32768;
+#pragma unroll
+				for (int i = 0; i < 8; i++)
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (a + source_offset[i]), (lds_ptr_t) (slot + (wave + 4 * i) * 1024), 16, 0, 2); /* non-temporal */
+			};
+			int frag_first[2];
+#pragma unroll
+			for (int rb = 0; rb < 2; rb++)
+			{
+				const int row = 32 * rb + frag_row;
+				frag_first[rb] = row * 128 + ((half_sel ^ ((row >> 1) & 7)) * 16);
+			}
+			if (my_chunks > 0)
+				request_chunk(0);
+			for (int ci = 0; ci < my_chunks; ci++)
+			{
+				wait_vmcnt<0>(); /* this chunk's A has landed (and the B operand, the first time) */
+				barrier_no_fence(); /* ... for every wavefront; nobody reads the other slot any more */
+				if (ci + 1 < my_chunks)
+					request_chunk(ci + 1);
+				const uint8_t *slot = lds + (ci & 1) * 32768;
+				acc_vec acc[2][2];
+#pragma unroll
+				for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+					for (int cg = 0; cg < 2; cg++)
+#pragma unroll
+						for (int r = 0; r < 16; r++)
+							acc[rb][cg][r] = 0;
+				uint4_t frags[2][2];
+#pragma unroll
+				for (int rb = 0; rb < 2; rb++)
+					frags[0][rb] = *reinterpret_cast<const uint4_t*>(slot + frag_first[rb]);
+				stream_static_for<16>([&](auto step)
+				{
+					constexpr int t = decltype(step)::value;
+					constexpr int cur = t & 1, nxt = 1 - cur;
+					if constexpr (t + 1 < 16)
+					{
+						constexpr int ks = (t + 1) / 4, kk = (t + 1) % 4;
+#pragma unroll
+						for (int rb = 0; rb < 2; rb++)
+							frags[nxt][rb] = *reinterpret_cast<const uint4_t*>(slot + ks * 8192 + (frag_first[rb] ^ (kk * 32)));
+					}
+#pragma unroll
+					for (int cg = 0; cg < 2; cg++)
+#pragma unroll
+						for (int rb = 0; rb < 2; rb++)
+							Traits::mma(b_regs[cg][t], frags[cur][rb], acc[rb][cg]);
+				});
+				/* the scratch copy this chunk goes to was last used by chunk ci - LAYER_BUFFERS: all its tasks must have read it */
+				if (threadIdx.x == 0)
+					s_word = (ci < LAYER_BUFFERS) ? 1u
+							: (wait_for_counter(&my.consumed[ci - LAYER_BUFFERS][0], LAYER_TASKS_PER_CHUNK, spin_limit) ? 1u : 0u);
+				__syncthreads();
+				if (s_word == 0)
+				{
+					if (threadIdx.x == 0)
+						__hip_atomic_fetch_add(errors, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					return;
+				}
+				/* lane l, register r of a block: m = 32 rb + l % 32, n = 64 wave + 32 cg + 8 (r / 4) + 4 (l / 32) + r % 4 */
+				half_t *dst = my_scratch + (static_cast<size_t>(ci % LAYER_BUFFERS) * 36 + p) * LAYER_CHUNK_TILES * LAYER_CHANNELS;
+#pragma unroll
+				for (int rb = 0; rb < 2; rb++)
+#pragma unroll
+					for (int cg = 0; cg < 2; cg++)
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+						{
+							uint2_t packed;
+							packed[0] = pack_rtz(acc[rb][cg][4 * q], acc[rb][cg][4 * q + 1]);
+							packed[1] = pack_rtz(acc[rb][cg][4 * q + 2], acc[rb][cg][4 * q + 3]);
+							*reinterpret_cast<uint2_t*>(dst + (32 * rb + frag_row) * LAYER_CHANNELS + wave * 64 + cg * 32 + 8 * q + 4 * half_sel) = packed;
+						}
+				wait_vmcnt<0>(); /* the L2 has this wavefront's stores */
+				__syncthreads(); /* ... and everyone's */
+				if (threadIdx.x == 0)
+					__hip_atomic_fetch_add(&my.produced[ci][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+			}
+		}
+		else
+		{
+			const int first_task = role - LAYER_GEMM_WORKGROUPS;
+			const int tasks = my_chunks * LAYER_TASKS_PER_CHUNK;
+			for (int task = first_task; task < tasks; task += LAYER_TRANSFORM_WORKGROUPS)
+			{
+				const int ci = task / LAYER_TASKS_PER_CHUNK;
+				const int sub = task - ci * LAYER_TASKS_PER_CHUNK;
+				const int image_in_chunk = sub >> 2;
+				__syncthreads(); /* the previous task has left the LDS image */
+				if (threadIdx.x == 0)
+					s_word = wait_for_counter(&my.produced[ci][0], LAYER_GEMM_WORKGROUPS, spin_limit) ? 1u : 0u;
+				__syncthreads();
+				if (s_word == 0)
+				{
+					if (threadIdx.x == 0)
+						__hip_atomic_fetch_add(errors, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+					return;
+				}
+				asm volatile("buffer_inv sc0" ::: "memory"); /* this CU's L1 may hold lines of an earlier chunk at the same addresses */
+				wait_vmcnt<0>();
+				const size_t image = static_cast<size_t>(xcd + LAYER_XCDS * ci) * 4 + image_in_chunk;
+				const size_t image_elements = static_cast<size_t>(height) * width * LAYER_CHANNELS;
+				FusedImage<half_t> g;
+				g.matrices = my_scratch + static_cast<size_t>(ci % LAYER_BUFFERS) * LAYER_CHUNK_ELEMENTS + image_in_chunk * 16 * LAYER_CHANNELS;
+				g.matrix_stride = static_cast<size_t>(LAYER_CHUNK_TILES) * LAYER_CHANNELS;
+				g.output = (output != nullptr) ? output + image * image_elements : nullptr;
+				g.ext = HAS_EXT ? ext + image * image_elements : nullptr;
+				g.bias = bias;
+				g.next_matrices = next_matrices + image * 16 * LAYER_CHANNELS;
+				g.next_stride = all_tiles * LAYER_CHANNELS;
+				g.act = act;
+				g.height = height;
+				g.width = width;
+				g.channels = LAYER_CHANNELS;
+				g.tiles_h = tiles_h;
+				g.tiles_w = tiles_w;
+				g.slice = sub & 3;
+				fused_transform_phase1<half_t, 4, 64, ACT, HAS_EXT, 256, true>(g, lds);
+				__syncthreads(); /* every thread has taken what it needs from the scratch copy */
+				if (threadIdx.x == 0)
+					__hip_atomic_fetch_add(&my.consumed[ci][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+				fused_transform_phase2<half_t, 4, 64, 256, true>(g, lds);
 			}
 		}
 	}
@@ -762,6 +1067,79 @@ namespace
 	}
 }
 
+namespace
+{
+	/* device word that counts workgroups of the whole-layer kernel that gave up waiting; one per device, never freed */
+	unsigned int* layer_error_word()
+	{
+		static std::mutex guard;
+		static std::map<int, unsigned int*> words;
+		std::lock_guard<std::mutex> lock(guard);
+		int device = 0;
+		MLHIP_CHECK(hipGetDevice(&device));
+		auto it = words.find(device);
+		if (it == words.end())
+		{
+			unsigned int *word = nullptr;
+			MLHIP_CHECK(hipMalloc(&word, sizeof(unsigned int)));
+			MLHIP_CHECK(hipMemset(word, 0, sizeof(unsigned int)));
+			it = words.insert(std::make_pair(device, word)).first;
+		}
+		return it->second;
+	}
+	bool layer_kernel_applies(const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlShape_t &shape, const mlTensor_t &bias,
+			const mlTensor_t &ext, const void *output, mlActivationType_t act)
+	{
+		const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; };
+		return input_matrices.dtype == DTYPE_FLOAT16 && shape.dim[3] == LAYER_CHANNELS && input_matrices.dim[2] == LAYER_CHANNELS
+				&& weight_matrices.dim[1] == LAYER_CHANNELS && weight_matrices.dim[2] == LAYER_CHANNELS
+				&& ceil_div(shape.dim[1], 4) * ceil_div(shape.dim[2], 4) == 16 && shape.dim[0] % 4 == 0 && shape.dim[0] >= 4 * LAYER_XCDS
+				&& shape.dim[0] <= 4 * LAYER_XCDS * LAYER_MAX_CHUNKS && (act == ACTIVATION_LINEAR || act == ACTIVATION_RELU)
+				&& aligned16(input_matrices.data) && aligned16(weight_matrices.data) && aligned16(bias.data) && aligned16(ext.data) && aligned16(output)
+				&& device_compute_units() == 256;
+	}
+	void launch_layer(mlContext_t context, const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlTensor_t &bias, const mlTensor_t &ext,
+			const mlShape_t &shape, void *output, mlActivationType_t act, mlTensor_t &next)
+	{
+		const hipStream_t stream = stream_of(context);
+		const size_t sync_bytes = sizeof(LayerSync) * LAYER_XCDS;
+		const size_t scratch_bytes = static_cast<size_t>(LAYER_XCDS) * LAYER_BUFFERS * LAYER_CHUNK_ELEMENTS * sizeof(half_t);
+		uint8_t *block = reinterpret_cast<uint8_t*>(get_workspace(context, sync_bytes + scratch_bytes));
+		LayerSync *sync = reinterpret_cast<LayerSync*>(block);
+		half_t *scratch = reinterpret_cast<half_t*>(block + sync_bytes);
+		unsigned int *errors = layer_error_word();
+		MLHIP_CHECK(hipMemsetAsync(sync, 0, sync_bytes, stream));
+		const int lds = 65536;
+		const dim3 grid(LAYER_XCDS * LAYER_WORKGROUPS_PER_XCD), block_dim(256);
+		const unsigned int spin_limit = 1u << 17; /* about a tenth of a second per wait before a workgroup gives up */
+#define MLHIP_LAUNCH_LAYER(ACT, EXT) \
+		do { \
+			auto kernel = kernel_winograd_layer_f16<ACT, EXT>; \
+			ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), lds); \
+			hipLaunchKernelGGL(kernel, grid, block_dim, lds, stream, ptr<const half_t>(input_matrices), ptr<const half_t>(weight_matrices), \
+					ptr<const half_t>(bias), ptr<const half_t>(ext), reinterpret_cast<half_t*>(output), ptr<half_t>(next), scratch, sync, errors, shape.dim[0], \
+					shape.dim[1], shape.dim[2], ceil_div(shape.dim[1], 4), ceil_div(shape.dim[2], 4), static_cast<int>(act), spin_limit); \
+		} while (0)
+		const bool relu = (act == ACTIVATION_RELU);
+		if (ext.data != nullptr)
+		{
+			if (relu)
+				MLHIP_LAUNCH_LAYER(1, true);
+			else
+				MLHIP_LAUNCH_LAYER(0, true);
+		}
+		else
+		{
+			if (relu)
+				MLHIP_LAUNCH_LAYER(1, false);
+			else
+				MLHIP_LAUNCH_LAYER(0, false);
+		}
+#undef MLHIP_LAUNCH_LAYER
+		MLHIP_CHECK(hipGetLastError());
+	}
+}
+
 extern "C"
 {
 	using namespace mlhip;
@@ -867,6 +1245,50 @@ extern "C"
 			launch_output_input<half_t, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
 		else
 			launch_output_input<float, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+	}
+	void hip_winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
+			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
+			mlTensor_t next_matrices)
+	{
+		MLHIP_REQUIRE(output_shape.rank == 4, "Winograd layer: output shape must be [B, H, W, C]");
+		require_supported(tile_size, input_matrices, input_matrices.dtype);
+		require_supported(tile_size, next_matrices, input_matrices.dtype);
+		MLHIP_REQUIRE(weight_matrices.rank == 3 && weight_matrices.dim[0] == 36 && weight_matrices.dtype == input_matrices.dtype
+				&& next_matrices.dtype == input_matrices.dtype, "Winograd layer: weight matrices must be [36, Cout, Cin] of the input's data type");
+		const size_t tiles = static_cast<size_t>(output_shape.dim[0]) * ceil_div(output_shape.dim[1], 4) * ceil_div(output_shape.dim[2], 4);
+		MLHIP_REQUIRE(static_cast<size_t>(input_matrices.dim[1]) == tiles && input_matrices.dim[2] == weight_matrices.dim[2]
+				&& weight_matrices.dim[1] == output_shape.dim[3] && static_cast<size_t>(next_matrices.dim[1]) == tiles
+				&& next_matrices.dim[2] == output_shape.dim[3], "Winograd layer: matrices must be [36, tiles, Cin], [36, Cout, Cin] and [36, tiles, Cout]");
+		if (tiles == 0 || output_shape.dim[3] == 0)
+			return;
+		MLHIP_REQUIRE(input_matrices.data != nullptr && weight_matrices.data != nullptr && next_matrices.data != nullptr, "Winograd layer: null tensor");
+		if (bias.data != nullptr)
+			MLHIP_REQUIRE(bias.dtype == input_matrices.dtype && volume(bias) == static_cast<size_t>(output_shape.dim[3]), "Winograd layer: bias must be [Cout]");
+		if (ext.data != nullptr)
+			MLHIP_REQUIRE(ext.dtype == input_matrices.dtype && volume(ext) == volume(output_shape), "Winograd layer: ext must have the output's shape and dtype");
+		if (layer_kernel_applies(input_matrices, weight_matrices, output_shape, bias, ext, output, act))
+		{
+			mlTensor_t next = next_matrices;
+			launch_layer(context, input_matrices, weight_matrices, bias, ext, output_shape, output, act, next);
+			return;
+		}
+		/* every other shape: the batched product into the caller's matrices, then the fused (or two-step) transform */
+		MLHIP_REQUIRE(output_matrices.data != nullptr && output_matrices.dtype == input_matrices.dtype && output_matrices.rank == 3
+				&& output_matrices.dim[0] == 36 && static_cast<size_t>(output_matrices.dim[1]) == tiles && output_matrices.dim[2] == output_shape.dim[3],
+				"Winograd layer: this shape needs output matrices [36, tiles, Cout] as intermediate storage");
+		hip_gemm_batched(context, input_matrices.dtype, shape_of(output_matrices), output_matrices.data, shape_of(input_matrices), input_matrices.data,
+				shape_of(weight_matrices), weight_matrices.data, 'n', 't', 1.0f, 0.0f);
+		hip_winograd_output_input_transform(context, tile_size, output_matrices, bias, ext, output_shape, output, act, next_matrices);
+	}
+	int hip_winograd_layer_errors(mlContext_t context)
+	{
+		MLHIP_CHECK(hipStreamSynchronize(stream_of(context)));
+		unsigned int *word = layer_error_word();
+		unsigned int count = 0;
+		MLHIP_CHECK(hipMemcpy(&count, word, sizeof(count), hipMemcpyDeviceToHost));
+		if (count != 0)
+			MLHIP_CHECK(hipMemset(word, 0, sizeof(count)));
+		return static_cast<int>(count);
 	}
 } /* extern "C" */
 

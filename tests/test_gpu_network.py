@@ -116,6 +116,10 @@ def test_full_size_batch_1024_properties(ctx):
     b = net.forward().copyToHost(ctx)
     assert mismatches(a, b) == 0
     assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0  # the benchmark's fused pass computes the same bits
+    net.fuse_layers = True  # whole layers as single launches (product kept in the L2 cache): the same bits again
+    assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0
+    assert ml.winogradLayerErrors(ctx) == 0
+    net.fuse_layers = False
     small = ResNet(ctx, 4, 15, 32, 256, 20, "float16", params, O.to_half)
     small.setInput(x[:4])
     c = small.forward().copyToHost(ctx)

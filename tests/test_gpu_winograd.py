@@ -195,3 +195,38 @@ def test_fused_output_input_transform_bit_exact(ctx, dtype, shape):
     ml.winogradOutputInputTransform(ctx, wshape, dm, shape, dy3, db, de, O.TANH, dv3)
     assert mismatches(dv3.copyToHost(ctx), dv2.copyToHost(ctx)) == 0
     assert mismatches(dy3.copyToHost(ctx), dy2.copyToHost(ctx)) == 0
+
+
+@pytest.mark.parametrize("case", [(32, 15, 15, True, True, O.RELU), (64, 13, 16, False, False, O.RELU), (36, 15, 15, True, False, O.LINEAR),
+                                  (256, 15, 15, True, True, O.RELU), (8, 15, 15, True, True, O.RELU), (32, 19, 19, True, True, O.RELU)])
+def test_whole_layer_launch_is_bit_identical(ctx, case):
+    """hip_winograd_layer_forward against the library's own batched product followed by the fused transform, bit for bit (the same MFMA
+    sequence per element), with and without residual / stored output, for batches that give the XCDs equal and unequal numbers of chunks.
+    The last two cases (batch below 32, 25 tiles per image) take the entry point's two-call route through the output matrices."""
+    batch, h, w, use_ext, keep_y, act = case
+    c = 256
+    rng = np.random.default_rng(batch + h)
+    tiles = batch * ((h + 3) // 4) * ((w + 3) // 4)
+    shape = (batch, h, w, c)
+    wshape = (c, 3, 3, c)
+    v = random_tensor(rng, (36, tiles, c), "float16")
+    u = random_tensor(rng, (36, c, c), "float16", 0.05)
+    bias = random_tensor(rng, (c,), "float16")
+    ext = random_tensor(rng, shape, "float16")
+    du, db, de = ml.toDevice(ctx, u), ml.toDevice(ctx, bias), ml.toDevice(ctx, ext)
+    # reference sequence of this library
+    dv, dm = ml.toDevice(ctx, v), ml.Tensor((36, tiles, c), "float16")
+    ml.gemmBatched(ctx, "n", "t", dm, dv, du, 1.0, 0.0)
+    want_y, want_next = ml.Tensor(shape, "float16"), ml.Tensor((36, tiles, c), "float16")
+    ml.winogradOutputInputTransform(ctx, wshape, dm, shape, want_y, db, de if use_ext else None, act, want_next)
+    # one launch, next matrices written over the input matrices as the network runner does
+    dv2, dm2 = ml.toDevice(ctx, v), ml.Tensor((36, tiles, c), "float16")
+    got_y = ml.Tensor(shape, "float16")
+    got_y.setall(ctx, 7.0)
+    for repeat in range(2):  # the second launch finds the scratch buffer and the counters used
+        ml.convertType(ctx, dv2, ml.toDevice(ctx, v))
+        ml.winogradLayerForward(ctx, wshape, dv2, du, dm2, shape, got_y if keep_y else None, db, de if use_ext else None, act, dv2)
+        assert ml.winogradLayerErrors(ctx) == 0
+        assert mismatches(dv2.copyToHost(ctx), want_next.copyToHost(ctx)) == 0
+        if keep_y:
+            assert mismatches(got_y.copyToHost(ctx), want_y.copyToHost(ctx)) == 0
