@@ -678,7 +678,9 @@ namespace
 	 * streaming product plus the fused transform take about 290 us. Measured reasons: only 28 of the 64 workgroups of an XCD transform,
 	 * and a task is a chain of latencies (about 14 us), so the transform side limits the pipeline; while a chunk of M waits for it, two
 	 * chunks' worth of streaming data pass through the 4 MiB L2 and evict about 80 % of M to HBM after all (HBM writes 548 MB per
-	 * launch where 302 MB are V'). A probe of the mechanism alone shows what is available: data ping-ponged between CUs of one XCD stays
+	 * launch where 302 MB are V'). With a single scratch copy (1.1 MiB resident) M does stay in the L2 (HBM traffic 665 MB per launch
+	 * against 1210 MB for the separate launches), but product and transform then alternate and the launch takes 520 us: the 4 MiB L2
+	 * cannot hold enough chunks in flight to cover the latency of a transform task. A probe of the mechanism alone shows what is available: data ping-ponged between CUs of one XCD stays
 	 * out of HBM (22 MB written for 3.4 GB exchanged), an XCD-wide barrier costs about 0.8 us, dropping the L1 costs little, whereas an
 	 * agent-scope acquire fence costs about 8 us.
 	 * ------------------------------------------------------------------------------------------------------------------- */
