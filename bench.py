@@ -40,10 +40,10 @@ CONFIGS = {
 }
 
 # HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each counter
-# scaled by its reading for a 256 MiB copy kernel in the same run (read 308.1 MiB + written 288.0 MiB).
+# scaled by its reading for a 256 MiB copy kernel in the same run (read 324.2 MiB + written 288.1 MiB).
 # Source: profiles/hbm_traffic_cfg2_resnet20x256_fp16_b1024.md
 MEASURED_GEMM_TRAFFIC_BYTES = {
-    "cfg2_resnet20x256_fp16_b1024": 625.1e6,
+    "cfg2_resnet20x256_fp16_b1024": 642.0e6,
 }
 
 

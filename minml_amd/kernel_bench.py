@@ -95,6 +95,19 @@ class Bench:
                      s * (36 * tiles * chans + pix * chans + chans))
             self.row("winograd", "winograd_output_transform +res", shape, lambda: ml.winogradOutputTransform(ctx, wshape, M, y, bias, x, "relu"),
                      s * (36 * tiles * chans + 2 * pix * chans + chans))
+            if chans % 64 == 0:
+                V2 = ml.Tensor((36, tiles, chans), dtype)
+                oshape = (batch, board, board, chans)
+                self.row("winograd", "winograd_output_input_transform", shape,
+                         lambda: ml.winogradOutputInputTransform(ctx, wshape, M, oshape, None, bias, None, "relu", V2), s * 2 * 36 * tiles * chans)
+                self.row("winograd", "winograd_output_input_transform +res, y", shape,
+                         lambda: ml.winogradOutputInputTransform(ctx, wshape, M, oshape, y, bias, x, "relu", V2),
+                         s * (2 * 36 * tiles * chans + 2 * pix * chans))
+                if tag == "cfg2":  # product and both transforms as one launch (experimental): priced with the bytes that must move
+                    self.row("winograd", "winograd_layer_forward (one launch)", shape,
+                             lambda: ml.winogradLayerForward(ctx, wshape, V, U, M, oshape, None, bias, None, "relu", V2),
+                             s * (2 * 36 * tiles * chans + 36 * chans * chans), 2.0 * 36 * tiles * chans * chans, dtype)
+                V2.free()
             for t in (x, y, w, bias, U, V, M):
                 t.free()
 
