@@ -75,7 +75,7 @@ def test_no_device_is_reported_not_hidden():
 
 
 def test_conv2d_algorithm_choice_and_workspace_contract():
-    """src/layers/Conv2D.cpp:141-191,450-530; sizes of SURVEY's cfg2: 36 * 16384 * 256 elements per matrices tensor."""
+    """src/layers/Conv2D.cpp:141-191,450-530; sizes of benchmark configuration 2: 36 * 16384 * 256 elements per matrices tensor."""
     c3 = Conv2D(None, (1024, 15, 15, 256), 256, 3, "relu", True, "float16")
     assert c3.forward_algorithm == WINOGRAD_NON_FUSED and c3.winograd_tile_size == 4
     assert get_matrices_shape(3, 4, (1024, 15, 15, 256)) == (36, 16384, 256)
@@ -148,7 +148,7 @@ def test_python_mirror_validates_before_calling_the_library():
 
 
 def test_flop_count_of_the_benchmark_network():
-    """SURVEY: 40 * 7.73e10 + 9.66e9 + 1.18e8 = 3.10e12 executed flops per batch of 1024 (cfg2)."""
+    """40 * 7.73e10 + 9.66e9 + 1.18e8 = 3.10e12 executed flops per batch of 1024 (benchmark configuration 2)."""
     net = ResNet.__new__(ResNet)
     net.batch, net.board, net.channels, net.blocks = 1024, 15, 256, 20
 
