@@ -169,3 +169,38 @@ def test_full_size_policy_and_value_inputs(ctx):
     out = ml.Tensor(x.shape, "float16")
     ml.batchnormInference(ctx, 1.0, dx, None, None, ml.toDevice(ctx, stats), 0.0, out, "linear")
     assert max_abs_rel(out.copyToHost(ctx), x) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_policy_and_value_heads_after_a_trunk(ctx, dtype):
+    """The two heads of a board-game network on one trunk output [B, 15, 15, 256], every step on the device against the same chain of
+    oracle calls: policy = 1x1 convolution to one plane -> softmax over the 225 squares; value = global average pooling -> Dense 256 ->
+    256 with ReLU -> Dense 256 -> 3 -> softmax (Dense rides on gemm_ex, as in the reference's src/layers/Dense.cpp)."""
+    rng = np.random.default_rng(21)
+    batch, board, c = 64, 15, 256
+    trunk = storage(np.maximum(rng.standard_normal((batch, board, board, c)), 0.0), dtype)
+    wp, bp = random_tensor(rng, (1, 1, 1, c), dtype, 0.1), random_tensor(rng, (1,), dtype)
+    w1, b1 = random_tensor(rng, (c, c), dtype, 0.1), random_tensor(rng, (c,), dtype)
+    w2, b2 = random_tensor(rng, (3, c), dtype, 0.1), random_tensor(rng, (3,), dtype)
+    dt = ml.toDevice(ctx, trunk)
+    # policy
+    logits = ml.Tensor((batch, board, board, 1), dtype)
+    ml.convolutionImplicitGemmForward(ctx, dt, ml.toDevice(ctx, wp), logits, ml.toDevice(ctx, bp), None, "linear")
+    policy = logits.view((batch, board * board))
+    ml.softmaxForward(ctx, policy, policy)
+    want_logits = O.conv2d_forward(trunk, wp, bp, None, O.LINEAR).reshape(batch, board * board)
+    want_policy = O.softmax_forward(want_logits)
+    assert max_abs_rel(policy.copyToHost(ctx), want_policy) <= TOL[dtype] * 2  # two chained steps
+    # value
+    pooled = ml.Tensor((batch, c), dtype)
+    ml.globalAveragePoolingForward(ctx, 1.0, dt, 0.0, pooled)
+    hidden = ml.Tensor((batch, c), dtype)
+    ml.gemm_ex(ctx, hidden, 1.0, "n", pooled, "t", ml.toDevice(ctx, w1), 0.0, None, ml.toDevice(ctx, b1), "relu")
+    out = ml.Tensor((batch, 3), dtype)
+    ml.gemm_ex(ctx, out, 1.0, "n", hidden, "t", ml.toDevice(ctx, w2), 0.0, None, ml.toDevice(ctx, b2), "linear")
+    ml.softmaxForward(ctx, out, out)
+    want = O.global_average_pooling_forward(trunk)
+    want = O.gemm(want, w1, bias=b1, act=O.RELU)
+    want = O.softmax_forward(O.gemm(want, w2, bias=b2))
+    assert max_abs_rel(out.copyToHost(ctx), want) <= TOL[dtype] * 4  # four chained steps
+    assert np.abs(O.as_float(out.copyToHost(ctx)).astype(np.float64).sum(axis=1) - 1.0).max() <= (1e-5 if dtype == "float32" else 3e-3)
