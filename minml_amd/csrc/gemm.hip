@@ -127,7 +127,7 @@ namespace mlhip
 		const bool plain = (g.alpha == 1.0f) && (g.beta == 0.0f) && (g.bias == nullptr) && (g.act == ACTIVATION_LINEAR) && (g.N * esize) % 16 == 0
 				&& aligned_to(g.D, 16) && ((g.stride_c * esize) % 16 == 0) && g.dtype != DTYPE_INT8;
 		if (fast && (g.stride_a != 0 || g.batch == 1)
-				&& (plain ? stream_gemm_plain_applies(g.M, g.batch, k_bytes, esize) : stream_gemm_applies(g.M, g.batch, k_bytes)))
+				&& ((plain || g.dtype == DTYPE_FLOAT16) ? stream_gemm_plain_applies(g.M, g.batch, k_bytes, esize) : stream_gemm_applies(g.M, g.batch, k_bytes)))
 		{
 			const StreamGemmArgs sg { g.A, g.B, g.D, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a, g.stride_b, g.stride_c };
 			bool launched = true;

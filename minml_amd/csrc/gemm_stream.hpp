@@ -428,10 +428,14 @@ namespace mlhip
 	{
 		return (k_bytes == 128 || k_bytes == 256 || k_bytes == 512) && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256;
 	}
-	/* the plain-store fp16 form is also instantiated for 768-byte rows (384 halfs), whose B operand still fits the registers */
+	/* the fp16 forms are also instantiated for 768-byte rows (384 halfs), whose B operand still fits the registers */
+	inline bool stream_gemm_half_applies(int M, int batch, size_t k_bytes)
+	{
+		return stream_gemm_applies(M, batch, k_bytes) || (k_bytes == 768 && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256);
+	}
 	inline bool stream_gemm_plain_applies(int M, int batch, size_t k_bytes, int element_size)
 	{
-		return stream_gemm_applies(M, batch, k_bytes) || (element_size == 2 && k_bytes == 768 && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256);
+		return (element_size == 2) ? stream_gemm_half_applies(M, batch, k_bytes) : stream_gemm_applies(M, batch, k_bytes);
 	}
 	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue>
 	inline void launch_stream_gemm_as(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
@@ -463,9 +467,13 @@ namespace mlhip
 	inline void launch_stream_gemm_kb(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
 	{
 		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
-		if (g.N > 128 && (PLAIN || KB < 512))
-			launch_stream_gemm_as<T, KB, 1, 8>(stream, g, epilogue);
-		else if (g.N > 128) /* 64 B-operand registers + side inputs + a 128-row accumulator do not fit 256 VGPRs: two column slices */
+		constexpr bool WIDE_FITS = PLAIN || KB < 512; /* else B-operand registers + side inputs + a 128-row accumulator exceed 256 VGPRs */
+		if (g.N > 128 && WIDE_FITS)
+		{
+			if constexpr (WIDE_FITS)
+				launch_stream_gemm_as<T, KB, 1, 8>(stream, g, epilogue);
+		}
+		else if (g.N > 128) /* column slices of 128: every row of A is then fetched by ceil(N / 128) workgroups of one XCD */
 			launch_stream_gemm_as<T, KB, 2, 4>(stream, g, epilogue);
 		else if (g.N > 64)
 			launch_stream_gemm_as<T, KB, 2, 4>(stream, g, epilogue);
@@ -487,7 +495,7 @@ namespace mlhip
 				launch_stream_gemm_kb<T, 512>(stream, g, epilogue);
 				break;
 			case 768:
-				if constexpr (std::is_same<Epilogue, PlainStore>::value && sizeof(T) == 2)
+				if constexpr (std::is_same<T, half_t>::value)
 				{
 					launch_stream_gemm_kb<T, 768>(stream, g, epilogue);
 					break;

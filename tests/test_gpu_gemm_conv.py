@@ -121,12 +121,13 @@ def test_gemm_ex_epilogue(ctx, dtype, act):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
-@pytest.mark.parametrize("k_bytes", [128, 256, 512])
+@pytest.mark.parametrize("k_bytes", [128, 256, 512, 768])
 @pytest.mark.parametrize("M,N", [(33001, 256), (32800, 100), (40000, 64), (33000, 28), (32769, 384)])
 def test_gemm_ex_streaming_shapes(ctx, dtype, k_bytes, M, N):
     """gemm_ex with short K rows and many rows of A (1x1 convolutions, dense heads): the persistent streaming kernel with the fused
     epilogue. All three wavefront layouts (N > 128, > 64, <= 64), column counts that are no multiple of 32, a ragged last row block,
-    more than 256 columns; bias + beta * C + ReLU, and a sigmoid in place."""
+    more than 256 columns; bias + beta * C + ReLU, and a sigmoid in place. 768-byte rows take this kernel in fp16 (384 channels) and the
+    tile engine in fp32."""
     K = k_bytes // (2 if dtype == "float16" else 4)
     rng = np.random.default_rng(M + N + k_bytes)
     A = random_tensor(rng, (M, K), dtype, 0.3)
