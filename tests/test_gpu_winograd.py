@@ -230,3 +230,25 @@ def test_whole_layer_launch_is_bit_identical(ctx, case):
         assert mismatches(dv2.copyToHost(ctx), want_next.copyToHost(ctx)) == 0
         if keep_y:
             assert mismatches(got_y.copyToHost(ctx), want_y.copyToHost(ctx)) == 0
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_residual_may_alias_the_output(ctx, dtype):
+    """y = act(transform + bias + y): the residual tensor is the output tensor itself (an in-place skip connection). Both the stand-alone
+    output transform and the fused form read every residual element before they write it."""
+    rng = np.random.default_rng(17)
+    shape, c = (3, 15, 15, 64), 64
+    tiles = 3 * 16
+    m = random_tensor(rng, (36, tiles, c), dtype)
+    bias = random_tensor(rng, (c,), dtype)
+    ext = random_tensor(rng, shape, dtype)
+    want_y = O.winograd_output_transform(m, shape, bias, ext, O.RELU)
+    dm, db = ml.toDevice(ctx, m), ml.toDevice(ctx, bias)
+    y = ml.toDevice(ctx, ext)
+    ml.winogradOutputTransform(ctx, (c, 3, 3, c), dm, y, db, y, O.RELU)
+    assert mismatches(y.copyToHost(ctx), want_y) == 0
+    y = ml.toDevice(ctx, ext)
+    nxt = ml.Tensor((36, tiles, c), dtype)
+    ml.winogradOutputInputTransform(ctx, (c, 3, 3, c), dm, shape, y, db, y, O.RELU, nxt)
+    assert mismatches(y.copyToHost(ctx), want_y) == 0
+    assert mismatches(nxt.copyToHost(ctx), O.winograd_input_transform(want_y)) == 0
