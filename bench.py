@@ -174,7 +174,17 @@ def main():
         if n_t:
             transforms["%s@%s" % (entry, label)] = {"kernel": kernel, "launches_timed": n_t, "avg_launch_us": t_t * 1e6, "algorithmic_bytes": nbytes,
                                                    "gbs": nbytes / t_t / 1e9, "frac_hbm": nbytes / t_t / 1e9 / PEAK_HBM_GBS}
-    kernel_name = "kernel_gemm_stream_wide_nt" if channels * esize == 512 else "kernel_gemm_nt"
+    kernel_name = "kernel_gemm_stream_wide_nt" if channels * esize in (128, 256, 512) else "kernel_gemm_dma"
+    # the roofline that bounds the dominant kernel: whichever of its algorithmic bytes and flops takes longer at the chip's peaks
+    hbm_bound = gemm_bytes / (PEAK_HBM_GBS * 1e9) >= gemm_flops / (PEAK_MFMA_TFLOPS[dtype] * 1e12)
+    if hbm_bound:
+        roofline = {"bound": "hbm", "achieved": gemm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gemm_gbs / PEAK_HBM_GBS}
+    else:
+        roofline = {"bound": "mfma", "achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s",
+                    "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype]}
+    roofline.update({"traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
+                     "kernel": "%s (36 batched Winograd GEMMs, M=%d N=K=%d)" % (kernel_name, tiles, channels),
+                     "algorithmic_bytes": gemm_bytes, "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6})
     result = {
         "metric": "positions/sec at batch 1024 (20x256 res-net fp16); % MFMA peak in conv GEMMs" if args.config.startswith("cfg2")
         else "positions/sec (%s)" % args.config,
@@ -184,10 +194,7 @@ def main():
         "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
                    "positions_per_launch": net.chunk, "cross_layer_transform_fusion": not args.unfused},
         "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
-        "roofline": {"bound": "hbm", "achieved": gemm_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gemm_gbs / PEAK_HBM_GBS,
-                     "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
-                     "kernel": "%s (36 batched Winograd GEMMs, M=%d N=K=%d)" % (kernel_name, tiles, channels),
-                     "algorithmic_bytes": gemm_bytes, "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6},
+        "roofline": roofline,
         "gemm_mfma": {"achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s", "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype],
                       "flops_per_launch": gemm_flops,
                       "hbm_limited_ceiling_frac": min(1.0, gemm_flops / gemm_bytes * PEAK_HBM_GBS * 1e9 / (PEAK_MFMA_TFLOPS[dtype] * 1e12))},
