@@ -168,6 +168,10 @@ namespace mlhip
 			{
 				Storage<T>::store(p, v[0]);
 			}
+			__device__ __forceinline__ void store_streaming(T *p) const
+			{
+				Storage<T>::store(p, v[0]);
+			}
 			__device__ __forceinline__ void zero()
 			{
 				v[0] = 0.0f;

@@ -115,7 +115,7 @@ namespace mlhip
 	 */
 	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue>
 	__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a,
-			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, Epilogue epilogue)
+			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, int sweep, Epilogue epilogue)
 	{
 		typedef StreamGemmConfig Cfg;
 		typedef MfmaTraits<T> Traits;
@@ -153,8 +153,18 @@ namespace mlhip
 		}
 		const int n0 = n_tile * BN + wave_n * 32; /* first column of this wavefront */
 		const int total_units = batch * tiles_m;
-		const int unit_begin = group * units_per_group;
-		const int unit_end = min(total_units, unit_begin + units_per_group);
+		/*
+		 * Which units this workgroup owns. Default: a contiguous range of units_per_group units, ascending. Sweep form (sweep > 0
+		 * workgroups per matrix): workgroup j of a matrix takes its row blocks j, j + sweep, ... and walks them from the last to the
+		 * first, so that all workgroups move through the rows of their matrices together, from the end to the beginning. A producer
+		 * that wrote these rows in ascending order left the last ones in the last-level cache, and a consumer that reads the product
+		 * in ascending order finds the rows written last by this kernel there.
+		 */
+		const int sweep_matrix = (sweep > 0) ? group / sweep : 0;
+		const int sweep_lane = (sweep > 0) ? group % sweep : 0;
+		const int unit_begin = (sweep > 0) ? sweep_matrix * tiles_m : group * units_per_group;
+		const int unit_end = (sweep > 0) ? ((sweep_matrix < batch && sweep_lane < tiles_m) ? unit_begin + 1 : unit_begin)
+				: min(total_units, unit_begin + units_per_group);
 		if (unit_begin >= unit_end)
 			return;
 
@@ -182,9 +192,11 @@ namespace mlhip
 			/* ---- a run of units of one matrix ---- */
 			const int matrix = unit / tiles_m;
 			const int run_end = min(unit_end, (matrix + 1) * tiles_m);
-			const int run_units = run_end - unit;
+			const int run_units = (sweep > 0) ? (tiles_m - sweep_lane + sweep - 1) / sweep : run_end - unit;
 			const int run_stages = run_units * STAGES_PER_UNIT;
-			const int first_tile = unit - matrix * tiles_m;
+			/* row block of the u-th unit of this run: tile_base + u * tile_step */
+			const int tile_base = (sweep > 0) ? sweep_lane + (run_units - 1) * sweep : unit - matrix * tiles_m;
+			const int tile_step = (sweep > 0) ? -sweep : 1;
 			const uint8_t *a_base = reinterpret_cast<const uint8_t*>(A + static_cast<size_t>(matrix) * stride_a);
 			const uint8_t *b_base = reinterpret_cast<const uint8_t*>(B + static_cast<size_t>(matrix) * stride_b);
 			T *c_base = C + static_cast<size_t>(matrix) * stride_c;
@@ -211,14 +223,14 @@ namespace mlhip
 			auto request_stage = [&](int g) __attribute__((always_inline))
 			{
 				const int u = g / STAGES_PER_UNIT, ks = g - u * STAGES_PER_UNIT;
-				const int m_first = (first_tile + u) * Cfg::BM;
+				const int m_first = (tile_base + u * tile_step) * Cfg::BM;
 				uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
 #pragma unroll
 				for (int i = 0; i < LOADS; i++)
 				{
 					const int m = min(m_first + load_row[i], M - 1); /* rows past the end re-read the last row; their products are never stored */
 					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * KB + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
-							(lds_ptr_t) (stage + (wave + WAVES * i) * 1024), 16, 0, 0);
+							(lds_ptr_t) (stage + (wave + WAVES * i) * 1024), 16, 0, 2); /* non-temporal: every row of A is read once */
 				}
 			};
 			uint4_t frags[2][BLOCKS];
@@ -265,7 +277,7 @@ namespace mlhip
 				{
 					if (!local.has_extra())
 						return;
-					const int m_first = (first_tile + u) * Cfg::BM + wave_m * ROWS;
+					const int m_first = (tile_base + u * tile_step) * Cfg::BM + wave_m * ROWS;
 #pragma unroll
 					for (int i = 0; i < BLOCKS; i++)
 #pragma unroll
@@ -278,7 +290,7 @@ namespace mlhip
 			auto store_unit = [&](int u) __attribute__((always_inline))
 			{
 				/* lane l, register r of block i: m = 32 i + l % 32, n = 8 (r / 4) + 4 (l / 32) + r % 4 */
-				const int m_first = (first_tile + u) * Cfg::BM + wave_m * ROWS;
+				const int m_first = (tile_base + u * tile_step) * Cfg::BM + wave_m * ROWS;
 				if constexpr (PLAIN)
 				{
 					constexpr int ELEMS_PER_16B = 16 / sizeof(T);
@@ -459,8 +471,19 @@ namespace mlhip
 		if (groups > total_units)
 			groups = total_units;
 		const int units_per_group = ceil_div(total_units, groups);
+		/*
+		 * Sweep form for batched products whose matrices each get at least two workgroups (the 36 Winograd matrices on 256 compute
+		 * units: 7 each, 252 workgroups): measured 1.3 % to 2.8 % more positions per second on the 20-block network than the
+		 * contiguous split, although it leaves 4 compute units idle, because the rows meet the last-level cache in the right order.
+		 */
+		int sweep = 0;
+		if (n_tiles == 1 && g.batch > 1 && groups / g.batch >= 2)
+		{
+			sweep = min(groups / g.batch, tiles_m);
+			groups = sweep * g.batch;
+		}
 		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
-				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, epilogue);
+				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, sweep, epilogue);
 	}
 	/* wavefront layout by output width: 8 x 32 columns for N > 128, 2 x 4 for N > 64, 4 x 2 below */
 	template<typename T, int KB, typename Epilogue>
