@@ -48,7 +48,10 @@ class ResNet:
         """params_host: list from make_parameters; to_storage: fp32 ndarray -> ndarray in the storage type (identity or fp16 bits)."""
         self.context = context
         self.fused = fused
-        self.fuse_block_boundary = True  # False: fuse only inside the residual blocks (for measurements)
+        # True: also fuse across the residual blocks' boundaries (the block's result is written and transformed for the next block in one
+        # launch). Identical results and less memory traffic, but measured 0.3 % to 1 % slower on MI355X than two launches there, whose
+        # second one finds the block's result in the last-level cache
+        self.fuse_block_boundary = False
         # True: whole layers (product + both transforms) as one launch that keeps the product in the L2 cache. Identical results, but
         # measured slower than the separate product and fused transform on MI355X (about 430 us against 290 us per layer at batch 1024),
         # so it is off unless asked for

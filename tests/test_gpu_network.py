@@ -99,10 +99,12 @@ def test_cross_layer_fusion_is_bit_identical(ctx, dtype, channels, blocks):
     net.setInput(x)
     plain = net.forward(fused=False).copyToHost(ctx)
     trunk_plain = net.trunk_output().copyToHost(ctx)
-    fused = net.forward(fused=True).copyToHost(ctx)
-    trunk_fused = net.trunk_output().copyToHost(ctx)
-    assert mismatches(plain, fused) == 0
-    assert mismatches(trunk_plain, trunk_fused) == 0
+    for across_blocks in (False, True):  # fusion inside the residual blocks only, then also across their boundaries
+        net.fuse_block_boundary = across_blocks
+        fused = net.forward(fused=True).copyToHost(ctx)
+        trunk_fused = net.trunk_output().copyToHost(ctx)
+        assert mismatches(plain, fused) == 0
+        assert mismatches(trunk_plain, trunk_fused) == 0
 
 
 def test_full_size_batch_1024_properties(ctx):
@@ -116,6 +118,8 @@ def test_full_size_batch_1024_properties(ctx):
     b = net.forward().copyToHost(ctx)
     assert mismatches(a, b) == 0
     assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0  # the benchmark's fused pass computes the same bits
+    net.fuse_block_boundary = True
+    assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0  # and so does fusion across the blocks' boundaries
     net.fuse_layers = True  # whole layers as single launches (product kept in the L2 cache): the same bits again
     assert mismatches(a, net.forward(fused=True).copyToHost(ctx)) == 0
     assert ml.winogradLayerErrors(ctx) == 0
