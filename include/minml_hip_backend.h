@@ -175,6 +175,18 @@ extern "C"
 	void hip_fold_batchnorm(mlContext_t context, mlTensor_t layer_weights, mlTensor_t layer_bias, const mlTensor_t bn_weights, const mlTensor_t bn_bias,
 			const mlTensor_t bn_avg_var); /* in place; rank-3 weights are depthwise (channels last), others channels first */
 
+	/* ---- transformer-block pieces of the hybrid networks: RMS normalisation and multi-head self-attention over the board's tokens with a
+	 *      2-D relative-position bias (reference: cuda_backend.h:199-200,207-210; arithmetic of the CPU backend:
+	 *      src/backend/cpu/normalization.cpp:452-486, src/backend/cpu/attention.cpp:142-214,395-431). fp16 and fp32, inference only. ---- */
+	void hip_rmsnorm_forward(mlContext_t context, mlShape_t shape, mlDataType_t dtype, const void *input, void *output,
+			const void *weights); /* rows of the last dim; weights (gamma) may be NULL */
+	int hip_multi_head_attention_get_workspace_size(mlShape_t input_shape, mlShape_t weights_shape, int num_heads,
+			bool training); /* elements; 0 for inference: the attention matrix never leaves the chip */
+	void hip_multi_head_attention_forward(mlContext_t context, mlShape_t input_shape, mlShape_t weights_shape, mlShape_t bias_shape, mlDataType_t dtype,
+			const void *input, void *output, const void *weights, const void *bias, void *workspace, void *backward_data, int num_heads,
+			bool symmetric); /* input [B,H,W,(3 - symmetric) E] = q,k,v per token; weights = position table [heads, 2r-1, round_up(2r-1, 4)] or NULL;
+			                    bias and workspace unused; backward_data must be NULL */
+
 	/* ---- additions with no counterpart in the reference ABI ----
 	 * hip_quantized_conv_forward: the whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 (int8 implicit GEMM with
 	 * zero-point padding, int32 accumulation, per-channel scale + bias, optional int8 residual, activation, requantisation)

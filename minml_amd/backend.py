@@ -101,6 +101,9 @@ SIGNATURES = {
     "global_average_pooling_forward": (None, [_vp, _f, _T, _f, _T]),
     "batchnorm_inference": (None, [_vp, _f, _T, _T, _T, _T, _f, _T, _i]),
     "fold_batchnorm": (None, [_vp, _T, _T, _T, _T, _T]),
+    "rmsnorm_forward": (None, [_vp, _S, _i, _vp, _vp, _vp]),
+    "multi_head_attention_get_workspace_size": (_i, [_S, _S, _i, _b]),
+    "multi_head_attention_forward": (None, [_vp, _S, _S, _S, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _b]),
     "quantized_conv_forward": (None, [_vp, _S, _S, _vp, _Q, _vp, _vp, _vp, _i, _vp, _Q, _vp, _Q, _i]),
     "get_stream": (_vp, [_vp]),
 }

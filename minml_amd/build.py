@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libminml_hip.so")
 
-SOURCES = ["runtime.hip", "winograd.hip", "gemm.hip", "conv.hip", "quantized.hip", "elementwise.hip", "heads.hip", "cuda_stubs.cpp"]
+SOURCES = ["runtime.hip", "winograd.hip", "gemm.hip", "conv.hip", "quantized.hip", "elementwise.hip", "heads.hip", "attention.hip", "cuda_stubs.cpp"]
 # packed fp32 VALU forms are switched off for all device code; the host pass does not know the feature and says so (harmless)
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

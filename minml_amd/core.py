@@ -523,6 +523,39 @@ def batchnormInference(context, alpha, input, weights, bias, avg_var, beta, outp
     _launch("batchnorm_inference", context.handle, alpha, input.desc(), _desc(weights), _desc(bias), avg_var.desc(), beta, output.desc(), act_of(act))
 
 
+def rmsnormForward(context, input, output, weights=None):
+    """y = (gamma * x) / (1e-6 + sqrt(mean x^2)) over the last dimension; weights (gamma) may be None (reference: src/core/math.cpp:844-860)."""
+    _require(_same_dtype(input, output, weights) and input.volume() == output.volume(), "shape / dtype mismatch")
+    _require(weights is None or weights.isEmpty() or weights.volume() == input.shape[-1], "weights must have one element per column")
+    _launch("rmsnorm_forward", context.handle, input.shape_desc(), input.dtype, input.ptr, output.ptr,
+            None if weights is None or weights.isEmpty() else weights.ptr)
+
+
+def multiHeadAttentionGetWorkspaceSize(context, input_shape, weights_shape, num_heads, training=False):
+    """Elements of workspace that multiHeadAttentionForward needs (reference: src/core/math.cpp:881-895)."""
+    return B.fn("multi_head_attention_get_workspace_size")(B.make_shape(input_shape), B.make_shape(weights_shape), num_heads, training)
+
+
+def multiHeadAttentionForward(context, input, output, weights, bias, workspace, backward_data, num_heads, symmetric):
+    """Self-attention over the H*W tokens of every image: input [B, H, W, (3 - symmetric) * E] holds q, k, v per token (k = q when
+    symmetric), weights is the relative-position table [heads, 2r-1, round_up(2r-1, 4)] or None, output [B, H, W, E]; bias and workspace
+    are accepted and unused, backward_data must be None or empty (reference: src/core/math.cpp:896-915)."""
+    parts = 2 if symmetric else 3
+    _require(len(input.shape) == 4 and input.shape[3] % parts == 0, "input must be [B, H, W, (3 - symmetric) * E]")
+    _require(tuple(output.shape) == tuple(input.shape[:3]) + (input.shape[3] // parts,) and _same_dtype(input, output, weights), "shape / dtype mismatch")
+    empty = lambda t: t is None or t.isEmpty()
+    _require((input.shape[3] // parts) % num_heads == 0, "embedding must be divisible by the number of heads")
+    _require(empty(backward_data), "keeping the attention matrix for a backward pass is not implemented (inference only)")
+    if not empty(weights):
+        size = weights.shape[1] if len(weights.shape) == 3 else 0
+        _require(len(weights.shape) == 3 and weights.shape[0] == num_heads and size % 2 == 1 and weights.shape[2] == (size + 3) // 4 * 4,
+                 "the position table must be [heads, 2r-1, round_up(2r-1, 4)]")
+    _launch("multi_head_attention_forward", context.handle, input.shape_desc(), B.make_shape(() if empty(weights) else weights.shape),
+            B.make_shape(() if empty(bias) else bias.shape), input.dtype, input.ptr, output.ptr, None if empty(weights) else weights.ptr,
+            None if empty(bias) else bias.ptr, None if empty(workspace) else workspace.ptr, None if empty(backward_data) else backward_data.ptr,
+            num_heads, bool(symmetric))
+
+
 def foldBatchnorm(context, layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
     """Folds a batch normalisation into the preceding layer's weights and bias, in place (reference: src/core/math.cpp:786-802, which
     also synchronises with the context afterwards)."""

@@ -57,11 +57,8 @@ MLHIP_STUB(cuda_batchnorm_backward)
 MLHIP_STUB(cuda_batchnorm_update)
 MLHIP_STUB(cuda_layernorm_forward)
 MLHIP_STUB(cuda_layernorm_backward)
-MLHIP_STUB(cuda_rmsnorm_forward)
 MLHIP_STUB(cuda_rmsnorm_backward)
 /* attention, mixture of experts */
-MLHIP_STUB(cuda_multi_head_attention_get_workspace_size)
-MLHIP_STUB(cuda_multi_head_attention_forward)
 MLHIP_STUB(cuda_multi_head_attention_backward)
 MLHIP_STUB(cuda_group_gemm)
 MLHIP_STUB(cuda_hash_routing)

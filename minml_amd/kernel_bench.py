@@ -8,7 +8,8 @@ achieved fraction of that peak.
 
 Groups: winograd (transforms and batched GEMM at the residual-network shapes), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
 channels 64..384, kernels 1 / 3 / 5, bias + residual + ReLU), int8 (quantised 3x3 convolution at 256 channels and its three-call form),
-misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode).
+misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode), transformer
+(RMS normalisation and multi-head attention at the hybrid configuration's shape).
 """
 import argparse
 import json
@@ -219,16 +220,35 @@ class Bench:
         for t in (x, y, pooled, gamma, bias, stats, logits, policy, many):
             t.free()
 
+    def transformer(self):
+        """The hybrid configuration's transformer block pieces: 256 images of 225 tokens, 8 heads of 32, fp16 (and the same in fp32)."""
+        ctx, rng = self.ctx, self.rng
+        batch, board, heads, head_dim = 256, 15, 8, 32
+        tokens, emb = board * board, heads * head_dim
+        for dtype, s in (("float16", 2), ("float32", 4)):
+            tag = "cfg5 B=256 15x15 8x32 " + ("f16" if s == 2 else "f32")
+            x = _random(ctx, (batch, board, board, emb), dtype, rng)
+            y = ml.Tensor((batch, board, board, emb), dtype)
+            gamma = _random(ctx, (emb,), dtype, rng)
+            self.row("transf.", "rmsnorm_forward", tag, lambda: ml.rmsnormForward(ctx, x, y, gamma), s * 2 * batch * tokens * emb)
+            qkv = _random(ctx, (batch, board, board, 3 * emb), dtype, rng)
+            table = _random(ctx, (heads, 2 * board - 1, 32), dtype, rng)
+            flops = 4.0 * batch * heads * tokens * tokens * head_dim  # q k^T and p v
+            self.row("transf.", "multi_head_attention_forward", tag, lambda: ml.multiHeadAttentionForward(ctx, qkv, y, table, None, None, None, heads, False),
+                     s * 4 * batch * tokens * emb, flops, dtype)
+            for t in (x, y, gamma, qkv, table):
+                t.free()
+
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
-    for group in ("winograd", "conv", "int8", "misc", "heads"):
+    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer"):
         if args.group in ("all", group):
             getattr(bench, group)()
     if args.json:

@@ -69,6 +69,8 @@ def lib():
         _lib.oracle_global_average_pooling_forward.argtypes = [_i, _i, _i, _i, _f, _c_void_p, _f, _c_void_p]
         _lib.oracle_batchnorm_inference.argtypes = [_i, _sz, _i, _f, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _f, _c_void_p, _i]
         _lib.oracle_fold_batchnorm.argtypes = [_i, _i, _i, _i, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p]
+        _lib.oracle_rmsnorm_forward.argtypes = [_i, _sz, _i, _c_void_p, _c_void_p, _c_void_p]
+        _lib.oracle_multi_head_attention_forward.argtypes = [_i, _i, _i, _i, _i, _i, _i, _c_void_p, _c_void_p, _c_void_p, _i]
     return _lib
 
 
@@ -279,6 +281,27 @@ def fold_batchnorm(layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
 # ---------------------------------------------------------------------------------------------------------------------------
 # the reference's own CPU backend, compiled from its sources by `make -C oracle ref` (present only where that was built)
 # ---------------------------------------------------------------------------------------------------------------------------
+def rmsnorm_forward(x, weights=None):
+    """y = (gamma * x) / (1e-6 + sqrt(mean x^2)) over the last dimension; `weights` (gamma, [last_dim]) may be None."""
+    x = _c(x)
+    w = None if weights is None else _c(weights)
+    out = np.empty_like(x)
+    lib().oracle_rmsnorm_forward(dtype_code(x), x.size // x.shape[-1], x.shape[-1], _p(x), _p(out), _p(w))
+    return out
+
+
+def multi_head_attention_forward(x, num_heads, table=None, symmetric=False):
+    """x [B, H, W, (3 - symmetric) * E] -> [B, H, W, E]; table [heads, 2r-1, round_up(2r-1, 4)] (relative-position bias) or None."""
+    x = _c(x)
+    t = None if table is None else _c(table)
+    b, h, w, c = x.shape
+    e = c // (2 if symmetric else 3)
+    out = np.empty((b, h, w, e), x.dtype)
+    lib().oracle_multi_head_attention_forward(dtype_code(x), b, h, w, e, num_heads, int(bool(symmetric)), _p(x), _p(out), _p(t),
+                                              0 if t is None else t.shape[1])
+    return out
+
+
 class _Shape(ctypes.Structure):
     _fields_ = [("rank", _i), ("dim", _i * 6)]
 
@@ -328,6 +351,8 @@ class Reference:
         L.cpu_softmax_forward.argtypes = [_c_void_p, _i, _Shape, _c_void_p, _c_void_p]
         L.cpu_global_average_pooling_forward.argtypes = [_c_void_p, _f, _Tensor, _f, _Tensor]
         L.cpu_fold_batchnorm.argtypes = [_c_void_p, _Tensor, _Tensor, _Tensor, _Tensor, _Tensor]
+        L.cpu_rmsnorm_forward.argtypes = [_c_void_p, _Shape, _i, _c_void_p, _c_void_p, _c_void_p]
+        L.cpu_multi_head_attention_forward.argtypes = [_c_void_p, _Tensor, _Tensor, _Tensor, _Tensor, _Tensor, _i]
         self.ctx = L.cpu_create_context()
 
     @staticmethod
@@ -436,6 +461,26 @@ class Reference:
         g, bb, st = _c(bn_weights, np.float32), _c(bn_bias, np.float32), _c(bn_avg_var, np.float32)
         self.lib.cpu_fold_batchnorm(self.ctx, _tensor(w), _tensor(b), _tensor(g), _tensor(bb), _tensor(st))
         return w, b
+
+
+    def rmsnorm_forward(self, x, weights=None):
+        """fp32 only (the reference has no other branch: normalization.cpp:460)."""
+        x = _c(x, np.float32)
+        w = None if weights is None else _c(weights, np.float32)
+        out = np.zeros_like(x)
+        self.lib.cpu_rmsnorm_forward(self.ctx, _shape(*x.shape), dtype_code(x), _p(x), _p(out), _p(w))
+        return out
+
+    def multi_head_attention_forward(self, x, num_heads, table=None):
+        """fp32 only; the layout (symmetric or not) follows from the channel count as in attention.cpp:408."""
+        x = _c(x, np.float32)
+        t = None if table is None else _c(table, np.float32)
+        b, h, w, c = x.shape
+        e = c // 3 if c % 3 == 0 else c // 2
+        out = np.zeros((b, h, w, e), np.float32)
+        workspace = np.zeros((b * num_heads * h * w * h * w,), np.float32)
+        self.lib.cpu_multi_head_attention_forward(self.ctx, _tensor(x), _tensor(out), _tensor(t), _tensor(workspace), _tensor(None), num_heads)
+        return out
 
 
 _ref = None

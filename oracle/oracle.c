@@ -739,3 +739,101 @@ void oracle_fold_batchnorm(int dtype, int channels, int other, int channels_last
 		}
 	}
 }
+
+/* ------------------------------------------------------------------------------------------------------------------------
+ * Transformer-block pieces: RMS normalisation and multi-head attention with a 2-D relative-position bias
+ * ---------------------------------------------------------------------------------------------------------------------- */
+/* src/backend/cpu/normalization.cpp:452-486: rms = sqrt(sum x^2 / n) with the sum taken in order, y = (gamma * x) * (1 / (1e-6 + rms)).
+ * The reference implements fp32 only; fp16 here widens on load and truncates on store like every other fp16 function. */
+void oracle_rmsnorm_forward(int dtype, size_t first_dim, int last_dim, const void *input, void *output, const void *weights)
+{
+#pragma omp parallel for num_threads(g_threads)
+	for (size_t i = 0; i < first_dim; i++)
+	{
+		float sum_square = 0.0f;
+		for (int j = 0; j < last_dim; j++)
+		{
+			const float x = load_as_float(input, i * last_dim + j, dtype);
+			const float sq = x * x;
+			sum_square = sum_square + sq;
+		}
+		const float rms = sqrtf(sum_square / (float) last_dim);
+		const float inv_rms = 1.0f / (1.0e-6f + rms);
+		for (int j = 0; j < last_dim; j++)
+		{
+			const float x = load_as_float(input, i * last_dim + j, dtype);
+			const float scaled = (weights != NULL) ? load_as_float(weights, j, dtype) * x : x;
+			store_from_float(output, i * last_dim + j, dtype, scaled * inv_rms);
+		}
+	}
+}
+
+/* src/backend/cpu/attention.cpp:395-431 (cpu_multi_head_attention_forward) with softmax_forward_in_place :142-214:
+ * input [B, H, W, (3 - symmetric) * E] holds per token q (heads x head_dim), k (absent when symmetric: k = q), v; per (b, head):
+ *   s[i][j] = (q_i . k_j, one fused multiply-add per element of the head in order) * (1 / sqrt(head_dim))        gemm 'n','t', :415-416
+ *   t[i][j] = s[i][j] + table[head][r + clamp(h_j - h_i, -r, r)][r + clamp(w_j - w_i, -r, r)],  r = (table_size - 1) / 2   :165-172
+ *   p[i][j] = exp(t[i][j] - max_j t[i][j]) * (1 / sum_j exp(...)), the sum taken in order                         :177-193
+ *   y[i][:] = sum_j p[i][j] * v_j, one fused multiply-add per j in order                                         gemm 'n','n', :423-424
+ * table is [heads][table_size][round_up(table_size, 4)] in the tensor's type, NULL for no bias. Output [B, H, W, E]. */
+void oracle_multi_head_attention_forward(int dtype, int batch, int height, int width, int embedding, int num_heads, int symmetric,
+		const void *input, void *output, const void *table, int table_size)
+{
+	const int tokens = height * width;
+	const int head_dim = embedding / num_heads;
+	const int parts = symmetric ? 2 : 3;
+	const size_t token_stride = (size_t) parts * embedding;
+	const float scale = (float) (1.0 / sqrt((double) head_dim)); /* :413 takes the root of an int: evaluated in double, then narrowed */
+	const int range = (table_size - 1) / 2;
+	const int table_row = (table_size + 3) / 4 * 4;
+#pragma omp parallel for collapse(2) num_threads(g_threads)
+	for (int b = 0; b < batch; b++)
+		for (int h = 0; h < num_heads; h++)
+		{
+			float *row = (float*) malloc(sizeof(float) * (size_t) tokens + 4);
+			float *acc = (float*) malloc(sizeof(float) * (size_t) head_dim + 4);
+			const size_t image = (size_t) b * tokens * token_stride;
+			const size_t q_off = image + (size_t) h * head_dim;
+			const size_t k_off = symmetric ? q_off : q_off + embedding;
+			const size_t v_off = q_off + (size_t) (parts - 1) * embedding;
+			for (int i = 0; i < tokens; i++)
+			{
+				const int h1 = i / width, w1 = i % width;
+				float max_value = -1.0e+32f;
+				for (int j = 0; j < tokens; j++)
+				{
+					float dot = 0.0f;
+					for (int d = 0; d < head_dim; d++)
+						dot = fmaf(load_as_float(input, q_off + i * token_stride + d, dtype), load_as_float(input, k_off + j * token_stride + d, dtype), dot);
+					float t = dot * scale;
+					if (table != NULL)
+					{
+						int dh = j / width - h1, dw = j % width - w1;
+						dh = (dh < -range) ? -range : ((dh > range) ? range : dh);
+						dw = (dw < -range) ? -range : ((dw > range) ? range : dw);
+						t = t + load_as_float(table, ((size_t) h * table_size + range + dh) * table_row + range + dw, dtype);
+					}
+					max_value = (t > max_value) ? t : max_value;
+					row[j] = t;
+				}
+				float sum = 0.0f;
+				for (int j = 0; j < tokens; j++)
+				{
+					row[j] = expf(row[j] - max_value);
+					sum = sum + row[j];
+				}
+				const float inv_sum = 1.0f / sum;
+				for (int d = 0; d < head_dim; d++)
+					acc[d] = 0.0f;
+				for (int j = 0; j < tokens; j++)
+				{
+					const float p = row[j] * inv_sum;
+					for (int d = 0; d < head_dim; d++)
+						acc[d] = fmaf(p, load_as_float(input, v_off + j * token_stride + d, dtype), acc[d]);
+				}
+				for (int d = 0; d < head_dim; d++)
+					store_from_float(output, ((size_t) b * tokens + i) * embedding + (size_t) h * head_dim + d, dtype, acc[d]);
+			}
+			free(row);
+			free(acc);
+		}
+}

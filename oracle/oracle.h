@@ -18,6 +18,12 @@
  *   int8_conv2d_forward   integer part against numpy int64; float tail against an independent numpy float32 evaluation and the
  *                         closed-form cases scale=1/shift=0; quantize() against the cases of test/backend/test_quantization.cpp:33-36
  *   fp16 conversion       exhaustive over all 65536 halfs (round trip) and against numpy with explicit truncation
+ *   rmsnorm_forward       float64 closed form, scale invariance, unit-norm rows; bit-exact agreement with oracle/_ref (fp32)
+ *   multi_head_attention_forward   float64 closed form; uniform attention for equal keys (output = mean of v); a table that forbids all
+ *                         but one offset (output = the v of that neighbour); bit-exact agreement with oracle/_ref (fp32). The fp16 form
+ *                         (fp16 in, fp32 arithmetic, truncated fp16 out) has no counterpart in the reference CPU backend, whose softmax
+ *                         reads the score matrix as fp32 whatever the tensor type (attention.cpp:420-426): it is pinned by the closed
+ *                         form only.
  */
 #ifndef MINML_ORACLE_H_
 #define MINML_ORACLE_H_
@@ -103,6 +109,14 @@ extern "C"
 	/* src/backend/cpu/normalization.cpp:296-343: batch normalisation folded into the preceding layer's weights and bias, in place */
 	void oracle_fold_batchnorm(int dtype, int channels, int other, int channels_last, void *layer_weights, void *layer_bias,
 			const void *bn_weights, const void *bn_bias, const float *bn_avg_var);
+
+	/* src/backend/cpu/normalization.cpp:452-486: y = (gamma * x) / (1e-6 + sqrt(mean x^2)) per row of [first_dim, last_dim]; gamma may be NULL */
+	void oracle_rmsnorm_forward(int dtype, size_t first_dim, int last_dim, const void *input, void *output, const void *weights);
+	/* src/backend/cpu/attention.cpp:142-214,395-431: softmax(q k^T / sqrt(head_dim) + relative-position bias) v per image and head;
+	 * input [B, H, W, (3 - symmetric) * E] (q, k, v per token; k = q when symmetric), output [B, H, W, E],
+	 * table [heads][table_size][round_up(table_size, 4)] or NULL */
+	void oracle_multi_head_attention_forward(int dtype, int batch, int height, int width, int embedding, int num_heads, int symmetric,
+			const void *input, void *output, const void *table, int table_size);
 
 #ifdef __cplusplus
 }

@@ -102,6 +102,15 @@ int main()
 	{	hip_convolution_implicit_gemm_forward(nullptr, DTYPE_INT8, shape(4, 1, 5, 5, 8), shape(4, 4, 3, 3, 8), buffer, buffer, buffer, nullptr, nullptr, ACTIVATION_RELU);}, "unsupported data type");
 	expect_throw<std::logic_error>("convert", [&]()
 	{	hip_convert_type(nullptr, buffer, DTYPE_INT32, buffer + 64, DTYPE_FLOAT32, 4);}, "unsupported conversion");
+	/* attention argument errors */
+	expect_throw<std::logic_error>("attention heads", [&]()
+	{	hip_multi_head_attention_forward(nullptr, shape(4, 1, 4, 4, 96), shape(0), shape(0), DTYPE_FLOAT32, buffer, buffer, nullptr, nullptr, nullptr, nullptr, 5, false);}, "divisible by the number of heads");
+	expect_throw<std::logic_error>("attention table", [&]()
+	{	hip_multi_head_attention_forward(nullptr, shape(4, 1, 4, 4, 96), shape(3, 4, 5, 5), shape(0), DTYPE_FLOAT32, buffer, buffer, buffer, nullptr, nullptr, nullptr, 4, false);}, "position table");
+	expect_throw<std::runtime_error>("attention training", [&]()
+	{	hip_multi_head_attention_forward(nullptr, shape(4, 1, 4, 4, 96), shape(0), shape(0), DTYPE_FLOAT32, buffer, buffer, nullptr, nullptr, nullptr, buffer, 4, false);}, "inference only");
+	expect_throw<std::logic_error>("rmsnorm dtype", [&]()
+	{	hip_rmsnorm_forward(nullptr, shape(2, 4, 8), DTYPE_INT8, buffer, buffer, nullptr);}, "unsupported data type");
 	/* valid arguments but no context */
 	expect_throw<std::logic_error>("null context", [&]()
 	{	hip_winograd_input_transform(nullptr, 4, tensor(buffer, DTYPE_FLOAT32, 4, 1, 4, 4, 2), tensor(buffer, DTYPE_FLOAT32, 3, 36, 1, 2));}, "null context");
@@ -119,6 +128,9 @@ int main()
 		hip_gemm(nullptr, DTYPE_FLOAT32, shape(2, 0, 4), nullptr, shape(2, 0, 8), nullptr, shape(2, 4, 8), buffer, 'n', 't', 1.0f, 0.0f);
 		(void) hip_get_number_of_devices();
 		(void) hip_supports_type(12345, DTYPE_FLOAT16);
+		hip_rmsnorm_forward(nullptr, shape(2, 0, 8), DTYPE_FLOAT32, nullptr, nullptr, nullptr);
+		if (hip_multi_head_attention_get_workspace_size(shape(4, 256, 15, 15, 768), shape(3, 8, 29, 32), 8, false) != 0)
+			throw std::runtime_error("inference attention asks for workspace");
 		hip_destroy_context(nullptr);
 		hip_destroy_event(nullptr);
 		hip_free(nullptr);

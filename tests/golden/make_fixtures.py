@@ -77,6 +77,14 @@ def main():
         folded_w, folded_b = ref.fold_batchnorm(fw, fb, gamma, beta, stats)
         out.update({key + "_w": fw, key + "_b": fb, key + "_gamma": gamma, key + "_beta": beta, key + "_stats": stats, key + "_w_out": folded_w,
                     key + "_b_out": folded_b})
+    # transformer-block pieces (the reference computes them in fp32 only): RMS normalisation with and without gamma; attention over a
+    # 5x7 board with 4 heads of 8 and a 5x5 position table (clamping active: offsets reach +-6), without table, and in the symmetric layout
+    rx, rg = init_for_test((9, 100), 0.0, 2.0), init_for_test((100,), 1.0) + np.float32(1.0)
+    out.update({"rms_x": rx, "rms_g": rg, "rms_y": ref.rmsnorm_forward(rx, rg), "rms_y_plain": ref.rmsnorm_forward(rx)})
+    ax, at = init_for_test((2, 5, 7, 96), 0.0, 1.5), init_for_test((4, 5, 8), 1.0)
+    ax2 = init_for_test((2, 4, 4, 64), 2.0, 1.5)
+    out.update({"mha_x": ax, "mha_table": at, "mha_y": ref.multi_head_attention_forward(ax, 4, at),
+                "mha_y_plain": ref.multi_head_attention_forward(ax, 4), "mha_sym_x": ax2, "mha_sym_y": ref.multi_head_attention_forward(ax2, 2)})
     # bit-plane unpacking and fp32 -> fp16 narrowing
     packed = (np.arange(3 * 5 * 2, dtype=np.uint64) * 2654435761 % (1 << 32)).astype(np.uint32)
     out["up_packed"] = packed

@@ -391,3 +391,74 @@ def test_batchnorm_inference_and_folding_agree():
     fdw, _ = O.fold_batchnorm(dw, b, gamma, beta, stats)
     scale = gamma / np.sqrt(stats[1].astype(np.float64) + 1e-6)
     assert np.abs(fdw - dw * scale).max() / np.abs(fdw).max() <= 1e-6
+
+
+def attention_float64(x, heads, table=None, symmetric=False):
+    """Textbook attention in float64 written from the definition: softmax(q k^T / sqrt(d) + bias) v per image and head."""
+    b, h, w, c = x.shape
+    parts = 2 if symmetric else 3
+    e = c // parts
+    d = e // heads
+    xs = x.astype(np.float64).reshape(b, h * w, parts, heads, d)
+    q, k, v = xs[:, :, 0], (xs[:, :, 0] if symmetric else xs[:, :, 1]), xs[:, :, parts - 1]
+    s = np.einsum("bihd,bjhd->bhij", q, k) / np.sqrt(d)
+    if table is not None:
+        r = (table.shape[1] - 1) // 2
+        rows, cols = np.divmod(np.arange(h * w), w)
+        dh = np.clip(rows[None, :] - rows[:, None], -r, r) + r  # [query, key]
+        dw = np.clip(cols[None, :] - cols[:, None], -r, r) + r
+        s = s + table.astype(np.float64)[:, dh, dw][None]
+    s = np.exp(s - s.max(axis=-1, keepdims=True))
+    p = s / s.sum(axis=-1, keepdims=True)
+    return np.einsum("bhij,bjhd->bihd", p, v).reshape(b, h, w, e)
+
+
+def test_rmsnorm_closed_form_and_invariants():
+    """Float64 closed form; rows leave with unit root-mean-square when gamma is absent; scaling a row by a positive constant changes
+    nothing (up to the 1e-6 in the denominator); a dropped square root, a sum instead of a mean or gamma applied twice fails the first."""
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal((13, 96)) * 3).astype(np.float32)
+    g = (rng.standard_normal(96) + 1.0).astype(np.float32)
+    rms = np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    assert np.abs(O.rmsnorm_forward(x, g) - g * x / (1e-6 + rms)).max() <= 2e-6 * np.abs(g).max() * 4
+    plain = O.rmsnorm_forward(x)
+    assert np.abs(np.sqrt((plain.astype(np.float64) ** 2).mean(axis=1)) - 1.0).max() <= 1e-5
+    assert np.abs(O.rmsnorm_forward(x * np.float32(8.0)) - plain).max() <= 1e-5
+    xh = O.to_half(x)
+    rms_h = np.sqrt((O.from_half(xh).astype(np.float64) ** 2).mean(axis=1, keepdims=True))
+    assert np.abs(O.as_float(O.rmsnorm_forward(xh)) - O.from_half(xh) / rms_h).max() <= 4e-3
+    assert np.array_equal(O.rmsnorm_forward(np.zeros((2, 8), np.float32)), np.zeros((2, 8), np.float32))  # 0 / (1e-6 + 0)
+
+
+@pytest.mark.parametrize("symmetric", [False, True])
+def test_attention_against_float64(symmetric):
+    rng = np.random.default_rng(12)
+    parts = 2 if symmetric else 3
+    x = rng.standard_normal((2, 4, 6, parts * 48)).astype(np.float32)
+    table = rng.standard_normal((3, 5, 8)).astype(np.float32)  # r = 3: offsets up to +-5 are clamped to +-2
+    for t in (None, table):
+        want = attention_float64(x, 3, t, symmetric)
+        assert np.abs(O.multi_head_attention_forward(x, 3, t, symmetric) - want).max() <= 1e-5
+    xh, th = O.to_half(x), O.to_half(table)
+    want = attention_float64(O.from_half(xh), 3, O.from_half(th), symmetric)
+    assert np.abs(O.as_float(O.multi_head_attention_forward(xh, 3, th, symmetric)) - want).max() <= 4e-3
+
+
+def test_attention_special_cases():
+    """(1) Equal keys give uniform attention: every output is the mean of the values. (2) A table that is hugely negative everywhere
+    except at one offset makes every token copy the value of the neighbour at that offset (tokens whose neighbour is off the board see
+    only clamped offsets and are skipped): pins the sign convention key - query, the row / column order of the table and the clamping."""
+    rng = np.random.default_rng(13)
+    b, h, w, heads, d = 2, 5, 6, 2, 8
+    e = heads * d
+    x = rng.standard_normal((b, h, w, 3, heads, d)).astype(np.float32)
+    x[:, :, :, 1] = x[0, 0, 0, 1]  # all keys equal
+    y = O.multi_head_attention_forward(x.reshape(b, h, w, 3 * e), heads)
+    mean_v = x[:, :, :, 2].astype(np.float64).mean(axis=(1, 2), keepdims=True)
+    assert np.abs(y.reshape(b, h, w, heads, d) - mean_v).max() <= 1e-6
+    x = rng.standard_normal((b, h, w, 3 * e)).astype(np.float32)
+    table = np.full((heads, 7, 8), -1.0e4, np.float32)  # r = 4 -> range 3
+    table[:, 3 + 1, 3 - 2] = 0.0  # key one row below, two columns to the left of the query
+    y = O.multi_head_attention_forward(x, heads, table).reshape(b, h, w, e)
+    v = x.reshape(b, h, w, 3, e)[:, :, :, 2]
+    assert np.abs(y[:, :h - 1, 2:] - v[:, 1:, :w - 2]).max() <= 1e-6

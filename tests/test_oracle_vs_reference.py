@@ -146,3 +146,31 @@ def test_reference_heads_bit_exact(dtype):
             stats = np.stack([rng.standard_normal(channels), rng.random(channels) + 0.05]).astype(np.float32)
             ours, theirs = O.fold_batchnorm(w, b, gamma, beta, stats), ref.fold_batchnorm(w, b, gamma, beta, stats)
             assert mismatches(ours[0], theirs[0]) == 0 and mismatches(ours[1], theirs[1]) == 0
+
+
+def test_fixtures_transformer_pieces(golden):
+    g = golden
+    assert mismatches(O.rmsnorm_forward(g["rms_x"], g["rms_g"]), g["rms_y"]) == 0
+    assert mismatches(O.rmsnorm_forward(g["rms_x"]), g["rms_y_plain"]) == 0
+    assert mismatches(O.multi_head_attention_forward(g["mha_x"], 4, g["mha_table"]), g["mha_y"]) == 0
+    assert mismatches(O.multi_head_attention_forward(g["mha_x"], 4), g["mha_y_plain"]) == 0
+    assert mismatches(O.multi_head_attention_forward(g["mha_sym_x"], 2, None, True), g["mha_sym_y"]) == 0
+
+
+@needs_ref
+def test_reference_transformer_pieces_bit_exact():
+    """fp32 only: the reference's RMS normalisation has no other branch and its attention reads the score matrix as fp32 whatever the type."""
+    ref = O.reference()
+    rng = np.random.default_rng(3)
+    for shape in ((7, 256), (3, 15, 15, 64), (5, 33), (2, 1)):
+        x, gamma = random_tensor(rng, shape, "float32", 2.0), random_tensor(rng, shape[-1:], "float32")
+        assert mismatches(O.rmsnorm_forward(x, gamma), ref.rmsnorm_forward(x, gamma)) == 0
+        assert mismatches(O.rmsnorm_forward(x), ref.rmsnorm_forward(x)) == 0
+    for (b, h, w, heads, d, r) in ((2, 15, 15, 2, 32, 8), (1, 6, 5, 3, 24, 3), (2, 3, 3, 1, 7, 1)):
+        x = random_tensor(rng, (b, h, w, 3 * heads * d), "float32")
+        size = 2 * r - 1
+        table = random_tensor(rng, (heads, size, (size + 3) // 4 * 4), "float32")
+        assert mismatches(O.multi_head_attention_forward(x, heads, table), ref.multi_head_attention_forward(x, heads, table)) == 0
+        assert mismatches(O.multi_head_attention_forward(x, heads), ref.multi_head_attention_forward(x, heads)) == 0
+    x = random_tensor(rng, (2, 5, 5, 2 * 4 * 16), "float32")
+    assert mismatches(O.multi_head_attention_forward(x, 4, None, True), ref.multi_head_attention_forward(x, 4)) == 0
