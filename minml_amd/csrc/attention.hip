@@ -89,13 +89,72 @@ namespace
 			}
 		}
 	}
+	/* the same with the row held in registers between the two passes: ITEMS vectors of VEC elements per lane, columns <= 64 * VEC * ITEMS */
+	template<typename T, int VEC, int ITEMS>
+	__global__ __launch_bounds__(256) void kernel_rmsnorm_in_registers(T *output, const T *input, const T *weights, size_t rows, int columns)
+	{
+		const int lane = threadIdx.x & 63;
+		const size_t stride = static_cast<size_t>(gridDim.x) * 4;
+		const float inv_columns = 1.0f / static_cast<float>(columns);
+		Vec<T, VEC> gamma[ITEMS];
+#pragma unroll
+		for (int i = 0; i < ITEMS; i++)
+		{
+			const int j = (lane + 64 * i) * VEC;
+#pragma unroll
+			for (int e = 0; e < VEC; e++)
+				gamma[i].v[e] = 1.0f;
+			if (weights != nullptr && j < columns)
+				gamma[i].load(weights + j);
+		}
+		for (size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6); row < rows; row += stride)
+		{
+			const T *src = input + row * columns;
+			T *dst = output + row * columns;
+			Vec<T, VEC> x[ITEMS];
+			float sum_square = 0.0f;
+#pragma unroll
+			for (int i = 0; i < ITEMS; i++)
+			{
+				const int j = (lane + 64 * i) * VEC;
+				x[i].zero();
+				if (j < columns)
+					x[i].load(src + j);
+#pragma unroll
+				for (int e = 0; e < VEC; e++)
+					sum_square = fmaf(x[i].v[e], x[i].v[e], sum_square);
+			}
+			sum_square = wave_sum(sum_square);
+			const float rms = sqrtf(sum_square * inv_columns);
+			const float inv_rms = 1.0f / (1.0e-6f + rms);
+#pragma unroll
+			for (int i = 0; i < ITEMS; i++)
+			{
+				const int j = (lane + 64 * i) * VEC;
+#pragma unroll
+				for (int e = 0; e < VEC; e++)
+					x[i].v[e] = (gamma[i].v[e] * x[i].v[e]) * inv_rms;
+				if (j < columns)
+					x[i].store(dst + j);
+			}
+		}
+	}
 	template<typename T>
 	void launch_rmsnorm(hipStream_t stream, T *output, const T *input, const T *weights, size_t rows, int columns)
 	{
 		constexpr int WIDE = 16 / sizeof(T);
 		const unsigned int groups = static_cast<unsigned int>(std::min<size_t>((rows + 3) / 4, 65536));
 		const bool aligned = (reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output) | reinterpret_cast<uintptr_t>(weights)) % 16 == 0;
-		if (columns % WIDE == 0 && aligned)
+		/* rows of up to 64 * WIDE * 4 elements stay in registers; the vector width shrinks for short rows so that all 64 lanes have work */
+		if (aligned && columns % WIDE == 0 && columns > 64 * WIDE / 2 && columns <= 64 * WIDE)
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 1>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+		else if (aligned && columns % WIDE == 0 && columns > 64 * WIDE && columns <= 64 * WIDE * 2)
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 2>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+		else if (aligned && columns % WIDE == 0 && columns > 64 * WIDE * 2 && columns <= 64 * WIDE * 4)
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 4>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+		else if (aligned && columns % (WIDE / 2) == 0 && columns <= 64 * WIDE / 2)
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE / 2, 1>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+		else if (aligned && columns % WIDE == 0)
 			hipLaunchKernelGGL((kernel_rmsnorm_forward<T, WIDE>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else
 			hipLaunchKernelGGL((kernel_rmsnorm_forward<T, 1>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
@@ -171,7 +230,17 @@ namespace
 			}
 	};
 
-	template<typename T, int D>
+	/* how the kernel finds a score's bias */
+	enum
+	{
+		BIAS_NONE = 0, /* no table */
+		BIAS_DIRECT = 1, /* the table spans every offset that occurs on the board (2r - 1 >= 2 max(H, W) - 1): no clamping, and the table index
+		 splits into a per-key and a per-query part, so that one addition per score finds the entry */
+		BIAS_CLAMPED = 2 /* offsets beyond the table's range use its border entries */
+	};
+	constexpr float LOG2_E = 1.4426950408889634f;
+
+	template<typename T, int D, int BIAS>
 	__global__ __launch_bounds__(256) void kernel_attention_mfma(const T *__restrict__ input, T *__restrict__ output, const T *__restrict__ table,
 			AttentionShape shape)
 	{
@@ -195,8 +264,9 @@ namespace
 		const int image = blockIdx.x / shape.heads;
 		const int head = blockIdx.x - image * shape.heads;
 		const T *tokens_base = input + static_cast<size_t>(image) * tokens * shape.token_stride + head * D;
-		const bool use_bias = shape.table_size > 0;
 		const int range = (shape.table_size - 1) / 2;
+		/* scores are kept in units of ln 2 (scale and table carry the factor log2 e) so that the exponential is the hardware's exp2 */
+		const float scale = shape.scale * LOG2_E;
 
 		/* ---- stage keys, transposed values, key places and the head's table ---- */
 		for (int i = threadIdx.x; i < tokens_padded * ROW_CHUNKS; i += 256)
@@ -229,14 +299,19 @@ namespace
 		}
 		for (int i = threadIdx.x; i < tokens_padded; i += 256)
 		{
-			const int row = i / shape.width;
-			place[i] = (static_cast<uint32_t>(row) << 16) | static_cast<uint32_t>(i - row * shape.width);
+			const int token = (i < tokens) ? i : 0; /* padding keys are masked later; they only need a harmless place */
+			const int row = token / shape.width;
+			const int column = token - row * shape.width;
+			if constexpr (BIAS == BIAS_DIRECT)
+				place[i] = static_cast<uint32_t>(row * shape.table_row + column) * 4u; /* the key's part of the entry's byte offset */
+			else
+				place[i] = (static_cast<uint32_t>(row) << 16) | static_cast<uint32_t>(column);
 		}
-		if (use_bias)
+		if constexpr (BIAS != BIAS_NONE)
 		{
 			const T *head_table = table + static_cast<size_t>(head) * shape.table_size * shape.table_row;
 			for (int i = threadIdx.x; i < shape.table_size * shape.table_row; i += 256)
-				bias[i] = Storage<T>::load(head_table + i);
+				bias[i] = Storage<T>::load(head_table + i) * LOG2_E;
 		}
 		__syncthreads();
 
@@ -259,8 +334,11 @@ namespace
 					q_frag[t] = *reinterpret_cast<const uint4_t*>(reinterpret_cast<const uint8_t*>(tokens_base + static_cast<size_t>(query) * shape.token_stride)
 							+ (2 * t + half_sel) * 16);
 			}
-			const int query_h = query / shape.width;
-			const int query_w = query - query_h * shape.width;
+			const int query_place = query_valid ? query : 0;
+			const int query_h = query_place / shape.width;
+			const int query_w = query_place - query_h * shape.width;
+			/* BIAS_DIRECT: entry (r + key_h - query_h, r + key_w - query_w) = this lane's base + the key's part */
+			const uint8_t *bias_base = reinterpret_cast<const uint8_t*>(bias) + ((range - query_h) * shape.table_row + (range - query_w)) * 4;
 
 			float running_max = -INFINITY, running_sum = 0.0f;
 			float16_t out[D_BLOCKS];
@@ -293,26 +371,35 @@ namespace
 #pragma unroll
 					for (int e = 0; e < 4; e++)
 					{
-						float value = s[4 * g + e] * shape.scale;
-						if (use_bias)
+						float value = s[4 * g + e] * scale;
+						if constexpr (BIAS == BIAS_DIRECT)
+							value = value + *reinterpret_cast<const float*>(bias_base + key_place[e]);
+						else if constexpr (BIAS == BIAS_CLAMPED)
 						{
 							const int dh = clamp_int(static_cast<int>(key_place[e] >> 16) - query_h, -range, range);
 							const int dw = clamp_int(static_cast<int>(key_place[e] & 0xffffu) - query_w, -range, range);
 							value = value + bias[(range + dh) * shape.table_row + range + dw];
 						}
-						value = (key0 + e < tokens) ? value : -INFINITY;
 						s[4 * g + e] = value;
-						block_max = fmaxf(block_max, value);
 					}
 				}
+				if (key_block == key_blocks - 1 && tokens != tokens_padded) /* the ragged last block: keys past the end do not take part */
+				{
+#pragma unroll
+					for (int r = 0; r < 16; r++)
+						s[r] = (key_block * 32 + 8 * (r / 4) + 4 * half_sel + (r % 4) < tokens) ? s[r] : -INFINITY;
+				}
+#pragma unroll
+				for (int r = 0; r < 16; r++)
+					block_max = fmaxf(block_max, s[r]);
 				block_max = fmaxf(block_max, __shfl_xor(block_max, 32));
 				const float new_max = fmaxf(running_max, block_max);
-				const float rescale = __expf(running_max - new_max);
+				const float rescale = __builtin_amdgcn_exp2f(running_max - new_max);
 				float block_sum = 0.0f;
 #pragma unroll
 				for (int r = 0; r < 16; r++)
 				{
-					s[r] = __expf(s[r] - new_max);
+					s[r] = __builtin_amdgcn_exp2f(s[r] - new_max);
 					block_sum += s[r];
 				}
 				block_sum += __shfl_xor(block_sum, 32);
@@ -447,10 +534,25 @@ namespace
 		const int bytes = Lds::bytes(shape.tokens, shape.table_size, shape.table_row);
 		if (bytes > MAX_ATTENTION_LDS)
 			return false;
-		const void *kernel = reinterpret_cast<const void*>(&kernel_attention_mfma<T, D>);
+		const int height = shape.tokens / shape.width;
+		const int bias = (shape.table_size == 0) ? BIAS_NONE : ((shape.table_size >= 2 * std::max(height, shape.width) - 1) ? BIAS_DIRECT : BIAS_CLAMPED);
+		const void *kernel = nullptr;
+		switch (bias)
+		{
+			case BIAS_NONE:
+				kernel = reinterpret_cast<const void*>(&kernel_attention_mfma<T, D, BIAS_NONE>);
+				break;
+			case BIAS_DIRECT:
+				kernel = reinterpret_cast<const void*>(&kernel_attention_mfma<T, D, BIAS_DIRECT>);
+				break;
+			default:
+				kernel = reinterpret_cast<const void*>(&kernel_attention_mfma<T, D, BIAS_CLAMPED>);
+				break;
+		}
 		ensure_dynamic_lds(kernel, bytes);
-		hipLaunchKernelGGL((kernel_attention_mfma<T, D>), dim3(batch * shape.heads), dim3(256), bytes, stream, input, output, table, shape);
-		MLHIP_CHECK(hipGetLastError());
+		AttentionShape shape_arg = shape;
+		void *args[] = { static_cast<void*>(&input), static_cast<void*>(&output), static_cast<void*>(&table), static_cast<void*>(&shape_arg) };
+		MLHIP_CHECK(hipLaunchKernel(kernel, dim3(batch * shape.heads), dim3(256), args, bytes, stream));
 		return true;
 	}
 	template<typename T>
