@@ -18,7 +18,8 @@
  *   int8_conv2d_forward   integer part against numpy int64; float tail against an independent numpy float32 evaluation and the
  *                         closed-form cases scale=1/shift=0; quantize() against the cases of test/backend/test_quantization.cpp:33-36
  *   fp16 conversion       exhaustive over all 65536 halfs (round trip) and against numpy with explicit truncation
- *   rmsnorm_forward       float64 closed form, scale invariance, unit-norm rows; bit-exact agreement with oracle/_ref (fp32)
+ *   rmsnorm_forward       float64 closed form, scale invariance, unit-norm rows; bit-exact agreement with oracle/_ref (fp32). The fp16 form
+ *                         has no counterpart in the reference CPU backend (normalization.cpp:460 has an fp32 branch only): closed form only.
  *   multi_head_attention_forward   float64 closed form; uniform attention for equal keys (output = mean of v); a table that forbids all
  *                         but one offset (output = the v of that neighbour); bit-exact agreement with oracle/_ref (fp32). The fp16 form
  *                         (fp16 in, fp32 arithmetic, truncated fp16 out) has no counterpart in the reference CPU backend, whose softmax
