@@ -142,3 +142,35 @@ def test_workspace_size_and_bad_arguments(ctx):
         ml.multiHeadAttentionForward(ctx, x, ml.Tensor((2, 4, 4, 32), "float32"), None, None, None, ml.Tensor((2 * 4 * 16 * 16,), "float32"), 4, False)
     with pytest.raises(ValueError):
         ml.rmsnormForward(ctx, x, ml.Tensor((2, 4, 4, 96), "float32"), ml.Tensor((95,), "float32"))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_attention_block_after_a_trunk(ctx, dtype):
+    """The attention half of a transformer block on a trunk output [B, 15, 15, 256], every step on the device against the same chain of
+    oracle calls: RMS normalisation -> Dense 256 -> 768 (q, k, v) -> attention with 8 heads and a full-range table -> Dense 256 -> 256
+    with the block's input as residual (Dense rides on gemm_ex with beta = 1, as the reference's fused Add does)."""
+    rng = np.random.default_rng(31)
+    batch, board, c, heads = 8, 15, 256, 8
+    rows = batch * board * board
+    trunk = random_tensor(rng, (batch, board, board, c), dtype)
+    gamma = random_tensor(rng, (c,), dtype, 0.2)
+    w_qkv, b_qkv = random_tensor(rng, (3 * c, c), dtype, 0.08), random_tensor(rng, (3 * c,), dtype, 0.1)
+    w_out, b_out = random_tensor(rng, (c, c), dtype, 0.08), random_tensor(rng, (c,), dtype, 0.1)
+    table = random_tensor(rng, (heads, 2 * board - 1, 32), dtype)
+    dt = ml.toDevice(ctx, trunk)
+    normed = ml.Tensor((batch, board, board, c), dtype)
+    ml.rmsnormForward(ctx, dt, normed, ml.toDevice(ctx, gamma))
+    qkv = ml.Tensor((batch, board, board, 3 * c), dtype)
+    ml.gemm_ex(ctx, qkv.view((rows, 3 * c)), 1.0, "n", normed.view((rows, c)), "t", ml.toDevice(ctx, w_qkv), 0.0, None, ml.toDevice(ctx, b_qkv), "linear")
+    mixed = ml.Tensor((batch, board, board, c), dtype)
+    ml.multiHeadAttentionForward(ctx, qkv, mixed, ml.toDevice(ctx, table), None, None, None, heads, False)
+    out = ml.Tensor((batch, board, board, c), dtype)
+    ml.gemm_ex(ctx, out.view((rows, c)), 1.0, "n", mixed.view((rows, c)), "t", ml.toDevice(ctx, w_out), 1.0, dt.view((rows, c)), ml.toDevice(ctx, b_out), "linear")
+    want = O.rmsnorm_forward(trunk, gamma)
+    assert max_abs_rel(normed.copyToHost(ctx), want) <= TOL[dtype]
+    want = O.gemm(want.reshape(rows, c), w_qkv, bias=b_qkv).reshape(batch, board, board, 3 * c)
+    assert max_abs_rel(qkv.copyToHost(ctx), want) <= TOL[dtype] * 2
+    want = O.multi_head_attention_forward(want, heads, table)
+    assert max_abs_rel(mixed.copyToHost(ctx), want) <= TOL[dtype] * 3
+    want = O.gemm(want.reshape(rows, c), w_out, beta=1.0, C=trunk.reshape(rows, c), bias=b_out).reshape(batch, board, board, c)
+    assert max_abs_rel(out.copyToHost(ctx), want) <= TOL[dtype] * 4  # four chained steps
