@@ -19,6 +19,10 @@ layer). Prints ONE JSON line:
   cpu_baseline the same network on a bounded number of positions on the host's cores: the reference's own CPU backend compiled from
                its sources (kind "reference", one thread, as the reference runs) when that library is present, otherwise this
                repository's C restatement (kind "port")
+
+--config cfg3_resnet20x256_int8_b1024 runs the int8 form of the same network instead (per-channel int8 weights, per-tensor int8
+activations calibrated on 64 random batches, every 3x3 layer one fused int8 implicit-GEMM convolution with int32 accumulation and
+requantisation); its roofline object prices that convolution against the dense int8 MFMA peak (5 POP/s).
 """
 import argparse
 import json
@@ -37,7 +41,10 @@ CONFIGS = {
     # name: (batch, board, input planes, channels, blocks, dtype, seed)
     "cfg2_resnet20x256_fp16_b1024": (1024, 15, 32, 256, 20, "float16", 1),
     "cfg1_resnet10x128_fp32_b256": (256, 15, 32, 128, 10, "float32", 0),
+    # the int8 form of configuration 2: same parameters (seed 1), per-channel int8 weights, per-tensor int8 activations calibrated on 64 batches
+    "cfg3_resnet20x256_int8_b1024": (1024, 15, 32, 256, 20, "int8", 1),
 }
+PEAK_INT8_TOPS = 5000.0
 
 # HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each counter
 # scaled by its reading for a 256 MiB copy kernel in the same run (read 324.2 MiB + written 288.1 MiB).
@@ -76,6 +83,82 @@ def run_cpu_baseline(params_storage, x_storage, blocks, budget_seconds):
             "sample": "%d positions of the same network and inputs, one forward pass, %.1f s" % (positions, t)}
 
 
+def run_int8_cpu_baseline(layers, blocks, x_int8, budget_seconds):
+    """The oracle's restatement of the reference's integer branch (the reference has no backend entry point for it: the arithmetic lives in
+    src/layers/Conv2D.cpp:240-308 and walks tensors element by element), multi-threaded, on as many positions as fit the budget."""
+    import oracle as O
+    from oracle.cpu_net import CpuQuantizedResNet
+
+    cores = min(16, os.cpu_count() or 1)
+    O.set_num_threads(cores)
+    net = CpuQuantizedResNet(layers, blocks)
+    positions = 1
+    t0 = time.perf_counter()
+    net.forward(x_int8[:positions])
+    t = time.perf_counter() - t0
+    target = int(max(1, min(x_int8.shape[0], budget_seconds / max(t, 1e-9))))
+    if target > positions:
+        positions = target
+        t0 = time.perf_counter()
+        net.forward(x_int8[:positions])
+        t = time.perf_counter() - t0
+    return {"value": positions / t, "unit": "positions/sec", "cores": cores, "kind": "port",
+            "sample": "%d positions of the same int8 network and inputs, one forward pass, %.1f s" % (positions, t)}
+
+
+def run_int8(args, ml):
+    """Configuration 3: the int8 network, every 3x3 layer one fused int8 implicit-GEMM convolution (--unfused: the reference's three calls)."""
+    from minml_amd import quantization as Q
+    from minml_amd.resnet import QuantizedResNet, calibrate_activations, make_input, make_parameters
+
+    batch, board, planes, channels, blocks, _, seed = CONFIGS[args.config]
+    params = make_parameters(seed, planes, channels, blocks)
+    x = make_input(seed, batch, board, planes)
+    ctx = ml.Context(0)
+    ranges = calibrate_activations(ctx, params, board, planes, channels, blocks, batches=64, batch_size=4, seed=seed)
+    net = QuantizedResNet(ctx, batch, board, planes, channels, blocks, params, ranges, "reference" if args.unfused else "fused")
+    net.setInput(x)
+    for _ in range(args.warmup):
+        net.forward()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.forward()
+    ctx.synchronize()
+    elapsed = time.perf_counter() - t0
+    timer = ml.KernelTimer(ctx)
+    ml.set_kernel_timer(timer)
+    for _ in range(max(1, min(args.steps, 5))):
+        net.forward()
+    kernels = timer.summary()
+    ml.set_kernel_timer(None)
+    entry = "gemm_v2" if args.unfused else "quantized_conv_forward"
+    count = sum(kernels.get(entry + "@" + l, (0, 0.0))[0] for l in ("block_conv1", "block_conv2"))
+    total = sum(kernels.get(entry + "@" + l, (0, 0.0))[0] * kernels.get(entry + "@" + l, (0, 0.0))[1] for l in ("block_conv1", "block_conv2"))
+    t_conv = total / count if count else float("nan")
+    pix = batch * board * board
+    conv_ops = 2.0 * pix * 9 * channels * channels
+    conv_bytes = pix * channels * 2.5 + 9 * channels * channels + 8 * channels  # int8 in, int8 out, the residual on every second layer
+    tops = conv_ops / t_conv / 1e12
+    result = {
+        "metric": "positions/sec (%s)" % args.config, "value": batch / (elapsed / args.steps), "unit": "positions/sec", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "i8",
+        "data": "synthetic (Bernoulli(0.3) input planes, He-normal weights quantised per output channel, activation ranges from 64 random "
+                "batches of 4 through the fp32 network, seed %d)" % seed,
+        "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
+                   "single_launch_int8_convolution": not args.unfused},
+        "tops_executed": net.ops_per_forward() / (elapsed / args.steps) / 1e12,
+        "roofline": {"bound": "mfma", "achieved": tops, "peak": PEAK_INT8_TOPS, "unit": "TOP/s", "frac": tops / PEAK_INT8_TOPS, "traffic": None,
+                     "kernel": ("int8 GEMM of the three-call form" if args.unfused else "kernel_gemm_dma<int8, im2row, requantisation>")
+                     + " (3x3 convolution as implicit GEMM, M=%d N=%d K=%d)" % (pix, channels, 9 * channels),
+                     "algorithmic_ops": conv_ops, "algorithmic_bytes": conv_bytes, "launches_timed": count, "avg_launch_us": t_conv * 1e6},
+    }
+    if args.cpu_seconds > 0:
+        result["cpu_baseline"] = run_int8_cpu_baseline(net.host_parameters, blocks, Q.quantize_tensor(x, net.transforms[0]), args.cpu_seconds)
+    print(json.dumps(result))
+
+
 def copy_calibration(ml, ctx):
     """One copy kernel of known size (256 MiB read, 256 MiB written) so that a counter run can be scaled against it."""
     n = 128 * 1024 * 1024
@@ -111,6 +194,8 @@ def main():
     from minml_amd import core as ml
     from minml_amd.resnet import ResNet, make_input, make_parameters, DEFAULT_CHUNK
 
+    if CONFIGS[args.config][5] == "int8":
+        return run_int8(args, ml)
     batch, board, planes, channels, blocks, dtype, seed = CONFIGS[args.config]
     chunk = args.chunk or DEFAULT_CHUNK.get(dtype, batch)
     to_storage = to_storage_factory(dtype)

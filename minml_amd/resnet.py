@@ -81,6 +81,12 @@ class ResNet:
     def setInput(self, x_storage):
         self.input.copyFromHost(self.context, x_storage)
 
+    def _observe(self, layer_index, tensor):
+        """Hands a layer's output to `self.observer(layer_index, tensor)` when one is set (layer-by-layer pass only); used for calibration
+        and per-layer checks."""
+        if getattr(self, "observer", None) is not None:
+            self.observer(layer_index, tensor)
+
     def _view_batch(self, tensor, start, count):
         per = tensor.volume() // tensor.shape[0]
         return tensor.view((count,) + tensor.shape[1:], start * per)
@@ -96,11 +102,14 @@ class ResNet:
             a, b, c = (self._view_batch(t, 0, n) for t in self.act)
             ml.set_timer_label("stem")
             self.layers[0].forward([x], a, self.workspace)
+            self._observe(0, a)
             for blk in range(self.blocks):
                 ml.set_timer_label("block_conv1")
                 self.layers[1 + 2 * blk].forward([a], b, self.workspace)
+                self._observe(1 + 2 * blk, b)
                 ml.set_timer_label("block_conv2")
                 self.layers[2 + 2 * blk].forward([b, a], c, self.workspace)
+                self._observe(2 + 2 * blk, c)
                 a, c = c, a
             ml.set_timer_label("head")
             self.layers[-1].forward([a], self._view_batch(self.output, start, n), self.workspace)
@@ -167,3 +176,91 @@ class ResNet:
             else:
                 total += 2 * self.batch * self.board * self.board * cin * cout * k * k
         return total
+
+
+def calibrate_activations(context, params_host, board, input_planes, channels, blocks, batches=64, batch_size=4, seed=0):
+    """Per-tensor activation ranges for the int8 network: max |x| of the input and of every 3x3 layer's output over `batches` random
+    batches, measured with the fp32 network on the device (benchmark configuration 3: "calibrated as the max-abs over 64 random batches").
+    Returns [input, stem, conv 1, ..., conv 2*blocks]."""
+    net = ResNet(context, batch_size, board, input_planes, channels, blocks, "float32", params_host, lambda a: np.ascontiguousarray(a, np.float32))
+    ranges = np.zeros(2 + 2 * blocks, np.float64)
+
+    def observer(index, tensor):
+        ranges[1 + index] = max(ranges[1 + index], float(np.abs(tensor.copyToHost(context)).max()))
+
+    net.observer = observer
+    for i in range(batches):
+        x = make_input(seed * 7919 + i + 1, batch_size, board, input_planes)
+        ranges[0] = max(ranges[0], float(np.abs(x).max()))
+        net.setInput(x)
+        net.forward(fused=False)
+    context.synchronize()
+    return [float(r) for r in ranges]
+
+
+class QuantizedResNet:
+    """The same network with int8 activations and weights (benchmark configuration 3): every 3x3 layer is one fused int8 convolution
+    (zero-point padding, int32 accumulation, per-channel scale + bias, int8 residual, ReLU, requantisation: src/layers/Conv2D.cpp:240-308),
+    the 1x1 head returns fp32 logits. Weights are quantised per output channel (scale = max|w| / 127), activations per tensor and
+    symmetric (scale = max|x| / 127 from `activation_ranges`, as returned by calibrate_activations)."""
+
+    def __init__(self, context, batch, board, input_planes, channels, blocks, params_host, activation_ranges, int8_mode="fused"):
+        from . import quantization as Q
+
+        self.context = context
+        self.batch, self.board, self.channels, self.blocks = batch, board, channels, blocks
+        self.transforms = [Q.symmetric_transform(r) for r in activation_ranges]  # input, stem, conv 1 ... conv 2*blocks
+        self.layers, self.host_parameters = [], []
+        shape = (batch, board, board, input_planes)
+        for index, (w, b) in enumerate(params_host):
+            head = index == len(params_host) - 1
+            layer = Conv2D(context, shape, w.shape[0], w.shape[1], "linear" if head else "relu", True, "int8")
+            in_qd = self.transforms[index]  # the tensor this layer reads was written by layer index - 1 (or is the input)
+            out_qd = (1.0, 0.0) if head else self.transforms[index + 1]
+            # the residual of a block's second convolution is the block's input: the output of the layer two steps back
+            ext_qd = self.transforms[index - 1] if (not head and index >= 2 and index % 2 == 0) else (1.0, 0.0)
+            q, scales, folded = Q.quantize_weights(w, b, in_qd)
+            layer.setupQuantization(q, scales, folded, [in_qd, ext_qd], out_qd, int8_mode)
+            self.layers.append(layer)
+            self.host_parameters.append((q, scales, folded, in_qd, ext_qd, out_qd))
+            shape = (batch, board, board, channels)
+        ws = max(1, max(l.getWorkspaceSize() for l in self.layers))
+        self.workspace = ml.Tensor((ws,), "float32", context.device_index)  # 4-byte elements, as Conv2D counts them in int8 mode
+        self.act = [ml.Tensor((batch, board, board, channels), "int8", context.device_index) for _ in range(3)]
+        self.input = ml.Tensor((batch, board, board, input_planes), "int8", context.device_index)
+        self.output = ml.Tensor((batch, board, board, 1), "float32", context.device_index)
+        self.observer = None
+
+    def setInput(self, x_real):
+        """Real-valued input planes -> int8 with the input's transform, uploaded."""
+        from . import quantization as Q
+
+        self.input.copyFromHost(self.context, Q.quantize_tensor(x_real, self.transforms[0]))
+
+    def forward(self):
+        L, ws = self.layers, self.workspace
+        a, b, c = self.act
+        ml.set_timer_label("stem")
+        L[0].forward([self.input], a, ws)
+        self._observe(0, a)
+        for blk in range(self.blocks):
+            ml.set_timer_label("block_conv1")
+            L[1 + 2 * blk].forward([a], b, ws)
+            self._observe(1 + 2 * blk, b)
+            ml.set_timer_label("block_conv2")
+            L[2 + 2 * blk].forward([b, a], c, ws)
+            self._observe(2 + 2 * blk, c)
+            a, c = c, a
+        ml.set_timer_label("head")
+        L[-1].forward([a], self.output, ws)
+        ml.set_timer_label(None)
+        return self.output
+
+    def _observe(self, layer_index, tensor):
+        if self.observer is not None:
+            self.observer(layer_index, tensor)
+
+    def ops_per_forward(self):
+        """Integer multiply-adds x 2 of one forward pass over the whole batch."""
+        pixels = self.batch * self.board * self.board
+        return sum(2 * pixels * int(np.prod(l.weight_shape)) for l in self.layers)

@@ -64,3 +64,29 @@ class CpuResNet:
             dt = time.perf_counter() - t0
             best = dt if best is None else min(best, dt)
         return best
+
+
+class CpuQuantizedResNet:
+    """The int8 form of the same network on the oracle's restatement of the reference's integer branch (src/layers/Conv2D.cpp:240-308):
+    every layer is oracle.int8_conv2d_forward with the layer's quantised weights, per-channel scales, folded bias and the three affine
+    transforms (input, residual, output). `layers` is a list of (q_weights, scales, bias, in_qd, ext_qd, out_qd), stem first, head last;
+    the head returns fp32."""
+
+    def __init__(self, layers, blocks):
+        self.layers = layers
+        self.blocks = blocks
+
+    def _conv(self, idx, x, ext, act, out_dtype=O.INT8):
+        q, scales, bias, in_qd, ext_qd, out_qd = self.layers[idx]
+        return O.int8_conv2d_forward(x, in_qd, q, scales, bias, out_dtype, out_qd, ext, ext_qd, act)
+
+    def forward(self, x_int8, per_layer=None):
+        a = self._conv(0, x_int8, None, O.RELU)
+        if per_layer is not None:
+            per_layer.append(a)
+        for blk in range(self.blocks):
+            t = self._conv(1 + 2 * blk, a, None, O.RELU)
+            a = self._conv(2 + 2 * blk, t, a, O.RELU)
+            if per_layer is not None:
+                per_layer.extend([t, a])
+        return self._conv(len(self.layers) - 1, a, None, O.LINEAR, O.FLOAT32)

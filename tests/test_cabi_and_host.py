@@ -159,3 +159,25 @@ def test_flop_count_of_the_benchmark_network():
     net.layers = [L((256, 3, 3, 32))] + [L((256, 3, 3, 256))] * 40 + [L((1, 1, 1, 256))]
     assert abs(net.flops_per_forward() - (40 * 2 * 36 * 16384 * 256 * 256 + 2 * 36 * 16384 * 32 * 256 + 2 * 230400 * 256)) < 1
     assert abs(net.flops_per_forward() / 3.10e12 - 1) < 0.01
+
+
+def test_host_side_quantisation_matches_the_oracle():
+    """minml_amd/quantization.py (what the product uses to prepare an int8 layer) against the oracle's restatement of the reference's
+    quantize / quantize_weights (src/layers/quantization.cpp:39-93), bit for bit, including halves (rounded away from zero) and clamping."""
+    import oracle as O
+    from minml_amd import quantization as Q
+
+    rng = np.random.default_rng(17)
+    x = np.concatenate([(rng.standard_normal(2000) * 60).astype(np.float32), np.array([0.5, -0.5, 1.5, 2.5, -2.5, 126.5, 127.5, -128.5, 1e9, -1e9], np.float32)])
+    assert np.array_equal(Q.quantize(x), np.array([O.quantize(float(v)) for v in x], np.int32))
+    for shape in ((44, 3, 3, 36), (64, 3, 3, 64), (7, 1, 1, 5)):
+        w = (rng.standard_normal(shape) * 0.1).astype(np.float32)
+        b = (rng.standard_normal(shape[0]) * 0.01).astype(np.float32)
+        for transform in ((0.031, 0.0), (0.02, -1.3)):
+            ours, theirs = Q.quantize_weights(w, b, transform), O.quantize_weights(w, b, transform)
+            for got, want in zip(ours, theirs):
+                assert np.array_equal(np.asarray(got).reshape(-1), np.asarray(want).reshape(-1))
+    values = (rng.standard_normal(500) * 3).astype(np.float32)
+    transform = Q.symmetric_transform(np.abs(values).max())
+    q = Q.quantize_tensor(values, transform)
+    assert q.dtype == np.int8 and np.abs(q.astype(np.int32)).max() == 127 and np.abs(q * np.float32(transform[0]) - values).max() <= transform[0] * 0.5001

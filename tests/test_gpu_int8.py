@@ -135,3 +135,37 @@ def test_int8_full_size_properties(ctx):
     total = int(acc.copyToHost(ctx).astype(np.int64).sum())
     colsum = x.reshape(-1, 256).astype(np.int64).sum(axis=0)
     assert total == int((w1.astype(np.int64) @ colsum).sum())
+
+
+@pytest.mark.parametrize("int8_mode", ["fused", "reference"])
+def test_quantized_network_bit_exact_per_layer_and_at_the_head(ctx, int8_mode):
+    """Configuration 3's recipe on a whole (small) network: activation ranges calibrated with the fp32 network, per-channel int8 weights,
+    every layer's int8 output and the fp32 head bit for bit against the oracle's integer branch, in the single-launch form and in the
+    reference's three-call form (im2row -> int8 GEMM -> requantisation)."""
+    from minml_amd import quantization as Q
+    from minml_amd.resnet import QuantizedResNet, calibrate_activations, make_input, make_parameters
+    from oracle.cpu_net import CpuQuantizedResNet
+
+    board, planes, channels, blocks, batch = 9, 32, 64, 3, 5
+    params = make_parameters(5, planes, channels, blocks)
+    ranges = calibrate_activations(ctx, params, board, planes, channels, blocks, batches=6, batch_size=3, seed=5)
+    assert len(ranges) == 2 + 2 * blocks and ranges[0] == 1.0 and all(r > 0 for r in ranges)
+    net = QuantizedResNet(ctx, batch, board, planes, channels, blocks, params, ranges, int8_mode)
+    # the host-side quantisation is the reference's (oracle restatement), bit for bit
+    for (w, b), (q, scales, folded, in_qd, _, _) in zip(params, net.host_parameters):
+        oq, oscales, ofolded = O.quantize_weights(w, b, in_qd)
+        assert np.array_equal(q.reshape(-1), np.asarray(oq).reshape(-1)) and np.array_equal(scales, oscales) and np.array_equal(folded, ofolded)
+    x = make_input(77, batch, board, planes)
+    xq = Q.quantize_tensor(x, net.transforms[0])
+    assert np.array_equal(xq, (x * 127).astype(np.int8))  # binary planes with range 1: scale 1 / 127, so the planes become 0 / 127
+    got_layers = []
+    net.observer = lambda index, tensor: got_layers.append(tensor.copyToHost(ctx))
+    net.setInput(x)
+    head = net.forward().copyToHost(ctx)
+    want_layers = []
+    want_head = CpuQuantizedResNet(net.host_parameters, blocks).forward(xq, want_layers)
+    assert len(got_layers) == len(want_layers) == 1 + 2 * blocks
+    for index, (got, want) in enumerate(zip(got_layers, want_layers)):
+        assert mismatches(got, want) == 0, "layer %d" % index
+        assert np.abs(got.astype(np.int32)).max() > 20  # the calibrated ranges are used, not a degenerate all-zero net
+    assert np.array_equal(head, want_head)
