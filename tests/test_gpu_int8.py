@@ -169,3 +169,32 @@ def test_quantized_network_bit_exact_per_layer_and_at_the_head(ctx, int8_mode):
         assert mismatches(got, want) == 0, "layer %d" % index
         assert np.abs(got.astype(np.int32)).max() > 20  # the calibrated ranges are used, not a degenerate all-zero net
     assert np.array_equal(head, want_head)
+
+
+def test_quantized_network_full_size(ctx):
+    """Configuration 3 itself (20 blocks x 256 channels, B = 1024): repeated passes give the same bits, the first positions reproduce a
+    batch-4 run of the same network bit for bit (positions are independent), and two of those positions match the oracle's integer
+    branch bit for bit at the fp32 head and at the last block's int8 output."""
+    from minml_amd import quantization as Q
+    from minml_amd.resnet import QuantizedResNet, calibrate_activations, make_input, make_parameters
+    from oracle.cpu_net import CpuQuantizedResNet
+
+    board, planes, channels, blocks = 15, 32, 256, 20
+    params = make_parameters(1, planes, channels, blocks)
+    ranges = calibrate_activations(ctx, params, board, planes, channels, blocks, batches=8, batch_size=4, seed=1)
+    x = make_input(1, 1024, board, planes)
+    net = QuantizedResNet(ctx, 1024, board, planes, channels, blocks, params, ranges)
+    net.setInput(x)
+    a = net.forward().copyToHost(ctx)
+    assert np.array_equal(a, net.forward().copyToHost(ctx))
+    assert np.isfinite(a).all() and np.abs(a).max() > 0
+    small = QuantizedResNet(ctx, 4, board, planes, channels, blocks, params, ranges)
+    small.setInput(x[:4])
+    trunk = []
+    small.observer = lambda index, tensor: trunk.append(tensor.copyToHost(ctx)) if index == 2 * blocks else None
+    b = small.forward().copyToHost(ctx)
+    assert np.array_equal(a[:4], b)
+    want_layers = []
+    want = CpuQuantizedResNet(small.host_parameters, blocks).forward(Q.quantize_tensor(x[:2], small.transforms[0]), want_layers)
+    assert np.array_equal(b[:2], want)
+    assert mismatches(trunk[0][:2], want_layers[-1]) == 0
