@@ -479,8 +479,12 @@ namespace mlhip
 		int sweep = 0;
 		if (n_tiles == 1 && g.batch > 1 && groups / g.batch >= 2)
 		{
-			sweep = min(groups / g.batch, tiles_m);
-			groups = sweep * g.batch;
+			const int per_matrix = min(groups / g.batch, tiles_m);
+			if ((groups - per_matrix * g.batch) * 16 <= groups) /* only when at most 1 / 16 of the compute units stay idle */
+			{
+				sweep = per_matrix;
+				groups = sweep * g.batch;
+			}
 		}
 		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
 				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, sweep, epilogue);
