@@ -174,3 +174,17 @@ def test_attention_block_after_a_trunk(ctx, dtype):
     assert max_abs_rel(mixed.copyToHost(ctx), want) <= TOL[dtype] * 3
     want = O.gemm(want.reshape(rows, c), w_out, beta=1.0, C=trunk.reshape(rows, c), bias=b_out).reshape(batch, board, board, c)
     assert max_abs_rel(out.copyToHost(ctx), want) <= TOL[dtype] * 4  # four chained steps
+
+
+def test_rmsnorm_full_size_properties(ctx):
+    """The hybrid configuration's tensor (256 x 15 x 15 tokens of 256 channels, fp16): without gamma every row leaves with unit
+    root-mean-square, scaling the input by a power of two changes no bit (up to the 1e-6 in the denominator), and a sample of rows
+    matches the oracle."""
+    rng = np.random.default_rng(4)
+    x = random_tensor(rng, (256, 15, 15, 256), "float16", 2.0)
+    y = rmsnorm(ctx, x)
+    values = O.as_float(y).astype(np.float64)
+    assert np.abs(np.sqrt((values ** 2).mean(axis=-1)) - 1.0).max() <= 2e-3  # truncation of 256 outputs per row
+    doubled = O.to_half(O.as_float(x) * np.float32(2.0))
+    assert mismatches(rmsnorm(ctx, doubled), y) <= y.size // 2000  # the 1e-6 moves a few results by one truncation step
+    assert max_abs_rel(y[7:9], O.rmsnorm_forward(x[7:9])) <= 1e-2
