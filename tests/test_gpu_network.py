@@ -186,3 +186,34 @@ def test_events_and_context(ctx):
     other.destroy()
     start.destroy()
     end.destroy()
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_network_driven_from_cpp_through_the_cabi(ctx, tmp_path, mode):
+    """The same network driven by a C++ program that includes only include/minml_hip_backend.h and links the library (tests/cabi_network.cpp:
+    descriptors by value from real C++, the reference's workspace layout, its call sequence per layer): the head output must equal the
+    Python mirror's bit for bit, in the three-call form and with the fused transform inside the residual blocks."""
+    import os
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    libdir = os.path.join(root, "minml_amd")
+    exe = str(tmp_path / "cabi_network")
+    subprocess.run(["g++", "-std=c++17", "-O2", "-o", exe, os.path.join(root, "tests", "cabi_network.cpp"), "-L" + libdir, "-lminml_hip",
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    batch, board, planes, channels, blocks = 6, 15, 32, 64, 3
+    params = make_parameters(12, planes, channels, blocks)
+    x = O.to_half(make_input(12, batch, board, planes))
+    with open(tmp_path / "parameters.bin", "wb") as f:
+        for w, b in params:
+            f.write(O.to_half(w).tobytes())
+            f.write(O.to_half(b).tobytes())
+    x.tofile(tmp_path / "input.bin")
+    res = subprocess.run([exe, str(tmp_path / "parameters.bin"), str(tmp_path / "input.bin"), str(tmp_path / "output.bin"), str(batch), str(board),
+                          str(planes), str(channels), str(blocks), str(mode), "3"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0 and "ALL OK" in res.stdout, res.stdout
+    got = np.fromfile(tmp_path / "output.bin", dtype=np.uint16).reshape(batch, board, board, 1)
+    net = ResNet(ctx, batch, board, planes, channels, blocks, "float16", params, O.to_half)
+    net.setInput(x)
+    want = net.forward(fused=bool(mode)).copyToHost(ctx)
+    assert mismatches(got, want) == 0
