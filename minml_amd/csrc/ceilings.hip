@@ -1,0 +1,192 @@
+/*
+ * ceilings.hip — probes of what one MI355X sustains, independent of the backend's kernels: plain read / write / copy streams over a
+ * buffer of a given size (HBM when the buffer exceeds the 256 MB last-level cache, that cache or the L2s when it fits) and a pure MFMA
+ * loop on operands held in registers. Built as its own small library (libminml_ceilings.so) and used only by
+ * `python3 -m minml_amd.kernel_bench --group ceilings`; nothing in the backend library depends on it.
+ *
+ * The entry points take a hipStream_t and raw device pointers and launch one kernel each; the caller times them with events.
+ */
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+
+namespace
+{
+	typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+	typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+	typedef float float16_t __attribute__((ext_vector_type(16)));
+	typedef int int16_t_v __attribute__((ext_vector_type(16)));
+	typedef int int4_v __attribute__((ext_vector_type(4)));
+
+	void check(hipError_t status, const char *what)
+	{
+		if (status != hipSuccess)
+			throw std::runtime_error(std::string("ceilings: ") + what + ": " + hipGetErrorString(status));
+	}
+
+	template<bool NT>
+	__device__ __forceinline__ uint4_t load16(const uint4_t *p)
+	{
+		return NT ? __builtin_nontemporal_load(p) : *p;
+	}
+	template<bool NT>
+	__device__ __forceinline__ void store16(uint4_t *p, uint4_t v)
+	{
+		if (NT)
+			__builtin_nontemporal_store(v, p);
+		else
+			*p = v;
+	}
+
+	/*
+	 * MODE 0: read `chunks` 16-byte pieces of src, 1: write them to dst, 2: copy src -> dst. Each workgroup owns a contiguous span;
+	 * within a span every instruction of a wavefront touches 1 KB of consecutive addresses, four instructions in flight per lane.
+	 */
+	template<int MODE, bool NT>
+	__global__ __launch_bounds__(256) void kernel_stream(uint4_t *__restrict__ dst, const uint4_t *__restrict__ src, size_t chunks, size_t chunks_per_wg)
+	{
+		const size_t begin = static_cast<size_t>(blockIdx.x) * chunks_per_wg;
+		const size_t end = (begin + chunks_per_wg < chunks) ? begin + chunks_per_wg : chunks;
+		uint32_t acc = 0;
+		size_t i = begin + threadIdx.x;
+		for (; i + 3 * 256 < end; i += 4 * 256)
+		{
+			uint4_t v[4];
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+			{
+				if (MODE != 1)
+					v[j] = load16<NT>(src + i + j * 256);
+				else
+					v[j] = uint4_t { static_cast<uint32_t>(i), 1u, 2u, static_cast<uint32_t>(j) };
+			}
+#pragma unroll
+			for (int j = 0; j < 4; j++)
+			{
+				if (MODE != 0)
+					store16<NT>(dst + i + j * 256, v[j]);
+				else
+					acc += v[j].x ^ v[j].w;
+			}
+		}
+		for (; i < end; i += 256)
+		{
+			uint4_t v = uint4_t { static_cast<uint32_t>(i), 1u, 2u, 3u };
+			if (MODE != 1)
+				v = load16<NT>(src + i);
+			if (MODE != 0)
+				store16<NT>(dst + i, v);
+			else
+				acc += v.x ^ v.w;
+		}
+		if (MODE == 0 && acc == 0x9e3779b9u && dst != nullptr)
+			dst[0] = uint4_t { acc, 0u, 0u, 0u };
+	}
+
+	/*
+	 * Pure matrix-pipe loop: every wavefront keeps 4 + 4 operand fragments in registers and issues 16 independent MFMAs per iteration
+	 * (a 128 x 128 sub-tile per k step, as a GEMM inner loop would, minus all memory traffic). RANDOM selects operand bits: all lanes
+	 * 1.0 (the pipes toggle little) or pseudo-random halfs / bytes in [-2, 2] (what real data looks like to the multipliers).
+	 * out[0..3] of workgroup 0 = shader-clock ticks and 100 MHz real-time ticks spent in the loop, for the clock the loop ran at.
+	 */
+	template<bool INT8>
+	__global__ __launch_bounds__(256, 1) void kernel_mfma_loop(uint64_t *out, int iters, int random)
+	{
+		const uint32_t lane = threadIdx.x;
+		uint4_t a[4], b[4];
+		for (int i = 0; i < 4; i++)
+			for (int j = 0; j < 4; j++)
+			{
+				const uint32_t h = (lane * 2654435761u) ^ ((i * 4 + j) * 40503u) ^ (blockIdx.x * 97u);
+				uint32_t word;
+				if (INT8)
+					word = random ? (h * 2246822519u) : 0x01010101u;
+				else
+				{
+					const uint32_t lo = 0x3000u | (h & 0x8fffu), hi = 0x3000u | ((h >> 16) & 0x8fffu);
+					word = random ? (lo | (hi << 16)) : 0x3c003c00u;
+				}
+				a[i][j] = word;
+				b[i][j] = word ^ (random ? 0x00010001u * (j + 1) : 0u);
+			}
+		float16_t accf[16];
+		int16_t_v acci[16];
+		for (int i = 0; i < 16; i++)
+			for (int r = 0; r < 16; r++)
+			{
+				accf[i][r] = 0.0f;
+				acci[i][r] = 0;
+			}
+		const uint64_t c0 = clock64();
+		const uint64_t w0 = wall_clock64();
+		for (int it = 0; it < iters; it++)
+		{
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+#pragma unroll
+				for (int j = 0; j < 4; j++)
+				{
+					if (INT8)
+						acci[i * 4 + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_v, b[j]), __builtin_bit_cast(int4_v, a[i]), acci[i * 4 + j],
+								0, 0, 0);
+					else
+						accf[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, b[j]), __builtin_bit_cast(half8_t, a[i]),
+								accf[i * 4 + j], 0, 0, 0);
+				}
+		}
+		const uint64_t c1 = clock64();
+		const uint64_t w1 = wall_clock64();
+		float s = 0.0f;
+		for (int i = 0; i < 16; i++)
+			for (int r = 0; r < 16; r++)
+				s += accf[i][r] + static_cast<float>(acci[i][r]);
+		if (blockIdx.x == 0 && threadIdx.x == 0)
+		{
+			out[0] = c1 - c0;
+			out[1] = w1 - w0;
+		}
+		if (s == 12345.678f)
+			out[2 + threadIdx.x] = static_cast<uint64_t>(s);
+	}
+}
+
+extern "C"
+{
+	/* mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16; nt != 0 uses non-temporal accesses */
+	void ceil_stream(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
+	{
+		if (bytes % 16 != 0 || workgroups <= 0 || mode < 0 || mode > 2)
+			throw std::logic_error("ceilings: ceil_stream: bad arguments");
+		const size_t chunks = bytes / 16;
+		size_t per_wg = (chunks + workgroups - 1) / workgroups;
+		per_wg = (per_wg + 1023) / 1024 * 1024; /* whole 16 KB blocks per workgroup */
+		const unsigned int grid = static_cast<unsigned int>((chunks + per_wg - 1) / per_wg);
+		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+		uint4_t *d = reinterpret_cast<uint4_t*>(dst);
+		const uint4_t *r = reinterpret_cast<const uint4_t*>(src);
+#define CEIL_LAUNCH(M, N) hipLaunchKernelGGL((kernel_stream<M, N>), dim3(grid), dim3(256), 0, s, d, r, chunks, per_wg)
+		switch (mode * 2 + (nt ? 1 : 0))
+		{
+			case 0: CEIL_LAUNCH(0, false); break;
+			case 1: CEIL_LAUNCH(0, true); break;
+			case 2: CEIL_LAUNCH(1, false); break;
+			case 3: CEIL_LAUNCH(1, true); break;
+			case 4: CEIL_LAUNCH(2, false); break;
+			default: CEIL_LAUNCH(2, true); break;
+		}
+#undef CEIL_LAUNCH
+		check(hipGetLastError(), "launch of kernel_stream");
+	}
+	/* one launch of the MFMA loop on `workgroups` workgroups of 4 wavefronts; `out` = at least 2 + 256 uint64 of device memory */
+	void ceil_mfma(void *stream, void *out, int iters, int random, int int8, int workgroups)
+	{
+		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+		if (int8)
+			hipLaunchKernelGGL(kernel_mfma_loop<true>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
+		else
+			hipLaunchKernelGGL(kernel_mfma_loop<false>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
+		check(hipGetLastError(), "launch of kernel_mfma_loop");
+	}
+}

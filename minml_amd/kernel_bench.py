@@ -9,10 +9,14 @@ achieved fraction of that peak.
 Groups: winograd (transforms and batched GEMM at the residual-network shapes), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
 channels 64..384, kernels 1 / 3 / 5, bias + residual + ReLU), int8 (quantised 3x3 convolution at 256 channels and its three-call form),
 misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode), transformer
-(RMS normalisation and multi-head attention at the hybrid configuration's shape).
+(RMS normalisation and multi-head attention at the hybrid configuration's shape), ceilings (what the chip sustains independent of the
+backend's kernels: read / write / copy streams over buffers that fit the L2s, the 256 MB last-level cache or neither, and a pure MFMA
+loop on constant and on random operands with the shader clock it ran at; needs libminml_ceilings.so, built by minml_amd.build).
 """
 import argparse
+import ctypes
 import json
+import os
 import sys
 
 import numpy as np
@@ -239,16 +243,88 @@ class Bench:
             for t in (x, y, gamma, qkv, table):
                 t.free()
 
+    def ceilings(self):
+        """Plain streams and a pure MFMA loop: the ceilings the other groups' rows can be read against."""
+        ctx = self.ctx
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libminml_ceilings.so")
+        if not os.path.exists(path):
+            raise RuntimeError("%s is missing: build it with `python -m minml_amd.build`" % path)
+        lib = ctypes.CDLL(path)
+        vp = ctypes.c_void_p
+        lib.ceil_stream.argtypes = [vp, vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.ceil_stream.restype = None
+        lib.ceil_mfma.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.ceil_mfma.restype = None
+        stream = ctx.stream()
+        mib = 1 << 20
+
+        def report(name, shape, t, nbytes):
+            gbs = nbytes / t / 1e9
+            r = {"group": "ceilings", "kernel": name, "shape": shape, "us": t * 1e6, "bound": "hbm", "achieved": gbs, "unit": "GB/s",
+                 "peak": PEAK["hbm"] / 1e9, "frac": gbs / (PEAK["hbm"] / 1e9), "algorithmic_MB": nbytes / 1e6, "algorithmic_Gop": 0.0}
+            self.rows.append(r)
+            print("%-9s %-34s %-34s %9.1f us  %-4s %9.1f %-7s  %5.1f %%" % ("ceilings", name, shape, r["us"], "hbm", gbs, "GB/s", 100 * r["frac"]),
+                  flush=True)
+
+        for size_mib, where in ((16, "fits the L2s"), (64, "fits the last-level cache"), (128, "fits the last-level cache"), (1024, "HBM")):
+            nbytes = size_mib * mib
+            a = ml.Tensor((nbytes,), "uint8")
+            b = ml.Tensor((nbytes,), "uint8")
+            a.zeroall(ctx)
+            b.zeroall(ctx)
+            wgs = 2048
+            shape = "%d MiB, %s" % (size_mib, where)
+            for nt in (0, 1):
+                tag = " (non-temporal)" if nt else ""
+                report("read stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, None, a.ptr, nbytes, 0, nt, wgs)), nbytes)
+                report("write stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, None, nbytes, 1, nt, wgs)), nbytes)
+                report("copy stream (read + write)" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, a.ptr, nbytes, 2, nt, wgs)), 2 * nbytes)
+            a.free()
+            b.free()
+        # producer -> consumer chains: launch i reads what launch i-1 wrote; three buffers in rotation
+        for size_mib in (32, 64, 512):
+            nbytes = size_mib * mib
+            bufs = [ml.Tensor((nbytes,), "uint8") for _ in range(3)]
+            for t in bufs:
+                t.zeroall(ctx)
+            state = {"i": 0}
+
+            def step():
+                i = state["i"]
+                lib.ceil_stream(stream, bufs[(i + 1) % 3].ptr, bufs[i % 3].ptr, nbytes, 2, 0, 2048)
+                state["i"] = i + 1
+
+            report("copy chain over 3 buffers", "3 x %d MiB" % size_mib, self.time(step), 2 * nbytes)
+            for t in bufs:
+                t.free()
+        out8 = ml.Tensor((4096,), "uint8")
+        iters, wgs = 20000, 256
+        for int8, name, peak, ops_per_mfma in ((0, "v_mfma_f32_32x32x16_f16", PEAK["float16"], 2.0 * 32 * 32 * 16),
+                                                (1, "v_mfma_i32_32x32x32_i8", PEAK["int8"], 2.0 * 32 * 32 * 32)):
+            for random in (0, 1):
+                t = self.time(lambda: lib.ceil_mfma(stream, out8.ptr, iters, random, int8, wgs))
+                ticks = out8.copyToHost(ctx).view(np.uint64)
+                clock_ghz = float(ticks[0]) / max(1.0, float(ticks[1])) * 0.1
+                ops = ops_per_mfma * 16 * iters * 4 * wgs
+                rate = ops / t
+                r = {"group": "ceilings", "kernel": name + " loop", "shape": "%s operands, %d CUs x 4 wavefronts" % ("random" if random else "constant", wgs),
+                     "us": t * 1e6, "bound": "mfma", "achieved": rate / 1e12, "unit": "TOP/s" if int8 else "TFLOP/s", "peak": peak / 1e12,
+                     "frac": rate / peak, "algorithmic_MB": 0.0, "algorithmic_Gop": ops / 1e9, "shader_clock_GHz": clock_ghz}
+                self.rows.append(r)
+                print("%-9s %-34s %-34s %9.1f us  %-4s %9.1f %-7s  %5.1f %%  shader clock %.2f GHz" % (
+                    "ceilings", r["kernel"], r["shape"], r["us"], "mfma", r["achieved"], r["unit"], 100 * r["frac"], clock_ghz), flush=True)
+        out8.free()
+
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "ceilings"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
-    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer"):
+    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer", "ceilings"):
         if args.group in ("all", group):
             getattr(bench, group)()
     if args.json:

@@ -26,10 +26,15 @@ _f = ctypes.c_float
 
 
 def build(reference="/root/reference"):
-    """Compiles liboracle.so, and oracle/_ref when a reference checkout is present."""
+    """Compiles liboracle.so and, when a reference checkout is present, oracle/_ref: the reference's CPU backend as a library, the
+    generator of the int8 layer fixtures, and (when the HIP library has been built) the reference's dispatcher, layers and graph linked
+    on top of the HIP library (`dropin_graph`, the link-time swap of the device backend)."""
     subprocess.run(["make", "-s", "-C", HERE, "oracle"], check=True)
     if os.path.isdir(os.path.join(reference, "src", "backend", "cpu")):
-        subprocess.run(["make", "-s", "-j8", "-C", HERE, "ref", "REF=" + reference], check=True)
+        targets = ["ref", "fixtures"]
+        if os.path.exists(os.path.join(HERE, "..", "minml_amd", "libminml_hip.so")):
+            targets.append("dropin")
+        subprocess.run(["make", "-s", "-j8", "-C", HERE] + targets + ["REF=" + reference], check=True)
 
 
 _lib = None

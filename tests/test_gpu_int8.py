@@ -198,3 +198,48 @@ def test_quantized_network_full_size(ctx):
     want = CpuQuantizedResNet(small.host_parameters, blocks).forward(Q.quantize_tensor(x[:2], small.transforms[0]), want_layers)
     assert np.array_equal(b[:2], want)
     assert mismatches(trunk[0][:2], want_layers[-1]) == 0
+
+
+def _reference_int8_cases():
+    import os
+
+    data = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_int8_conv2d.npz"))
+    return data, sorted({k.split("/")[0] for k in data.files})
+
+
+_REF8, _REF8_NAMES = _reference_int8_cases()
+
+
+@pytest.mark.parametrize("name", _REF8_NAMES)
+def test_int8_convolution_equals_reference_layer(ctx, name):
+    """Both device routes against what the reference's own Conv2D::forward (integer branch, src/layers/Conv2D.cpp:240-308) and
+    quantize_weights produced (tests/golden/make_int8_fixtures.py): bit for bit for linear / ReLU, int8 and fp32 outputs; for sigmoid /
+    tanh / exp the device's exponential differs from the host libm in the last place, so int8 outputs may differ by one count and fp32
+    outputs by 1e-6 relative."""
+    spec = [int(v) for v in _REF8[name + "/spec"]]
+    qd = [float(v) for v in _REF8[name + "/qd"]]
+    b, h, w, cin, cout, k, act, has_ext, int8_out = spec
+    in_qd, out_qd, ext_qd = (qd[0], qd[1]), (qd[2], qd[3]), (qd[4], qd[5])
+    x, q, scales, folded, want = (_REF8[name + "/" + key] for key in ("x", "q", "scales", "folded_bias", "y"))
+    de = ml.toDevice(ctx, _REF8[name + "/ext"]) if has_ext else None
+    dx, dw, ds, db = (ml.toDevice(ctx, a) for a in (x, q, scales, folded))
+    exact = act in (O.LINEAR, O.RELU)
+
+    def check(got):
+        if exact:
+            assert mismatches(got, want) == 0
+        elif int8_out:
+            assert np.abs(got.astype(np.int32) - want.astype(np.int32)).max() <= 1
+        else:
+            assert np.abs(got - want).max() <= 1e-6 * max(1.0, np.abs(want).max())
+
+    dy = ml.Tensor((b, h, w, cout), "int8" if int8_out else "float32")
+    ml.quantizedConvForward(ctx, dx, in_qd, dw, ds, db, dy, out_qd, de, ext_qd, act)
+    check(dy.copyToHost(ctx))
+    if int8_out:  # the reference's three device calls (im2row with the zero-point padding, int8 GEMM, requantisation)
+        layer = Conv2D(ctx, (b, h, w, cin), cout, k, act, True, "int8")
+        layer.setupQuantization(q, scales, folded, [in_qd, ext_qd], out_qd, int8_mode="reference")
+        ws = ml.Tensor((max(1, layer.getWorkspaceSize()),), B.DTYPE_INT32)
+        dy2 = ml.Tensor((b, h, w, cout), "int8")
+        layer.forward([dx, de] if has_ext else [dx], dy2, ws)
+        check(dy2.copyToHost(ctx))
