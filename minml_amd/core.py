@@ -154,6 +154,15 @@ class Tensor:
                 context.synchronize()  # the host array may go away
         return self
 
+    def copyFrom(self, context, other):
+        """Device-to-device copy of `other` into this tensor, asynchronous on the context's stream (reference: Tensor::copyFrom,
+        src/core/Tensor.cpp -> ml::memcpy -> cuda_memcpy_within_device)."""
+        if other.sizeInBytes() != self.sizeInBytes():
+            raise ValueError("copyFrom: sizes differ")
+        if self.sizeInBytes():
+            B.fn("memcpy_within_device")(context.handle if context else None, self.ptr, 0, other.ptr, 0, self.sizeInBytes())
+        return self
+
     def copyToHost(self, context=None):
         out = np.empty(self.shape, _NP_OF[self.dtype])
         if out.size:

@@ -62,7 +62,8 @@ namespace mlhip
 	void* get_workspace(mlContext_t context, size_t bytes);
 	/* number of compute units of the current device (cached per device) */
 	int device_compute_units();
-	/* opts a kernel in to `bytes` of dynamic LDS (more than the 64 KB default) on the current device; remembered per device and kernel */
+	/* makes sure a kernel may be launched with `bytes` of dynamic LDS on the current device (requests above the 64 KB default raise the
+	 * kernel's limit; the largest size granted so far is remembered per device and kernel) */
 	void ensure_dynamic_lds(const void *kernel, int bytes);
 
 	inline int size_of(mlDataType_t dtype)

@@ -6,7 +6,7 @@
 
 #include <cstring>
 #include <mutex>
-#include <set>
+#include <map>
 #include <sstream>
 #include <string>
 #include <utility>
@@ -117,13 +117,22 @@ namespace mlhip
 	}
 	void ensure_dynamic_lds(const void *kernel, int bytes)
 	{
+		/* largest size granted so far per (device, kernel): callers ask for shape-dependent sizes, so a later, larger request must raise
+		 * the limit again; the limit never goes below the 64 KB every kernel has by default */
 		static std::mutex guard;
-		static std::set<std::pair<int, const void*>> configured;
+		static std::map<std::pair<int, const void*>, int> granted;
+		constexpr int DEFAULT_LIMIT = 64 * 1024;
+		if (bytes <= DEFAULT_LIMIT)
+			return;
 		int device = 0;
 		MLHIP_CHECK(hipGetDevice(&device));
 		std::lock_guard<std::mutex> lock(guard);
-		if (configured.insert(std::make_pair(device, kernel)).second)
+		int &limit = granted[std::make_pair(device, kernel)];
+		if (bytes > limit)
+		{
 			MLHIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+			limit = bytes;
+		}
 	}
 	void* get_workspace(mlContext_t context, size_t bytes)
 	{

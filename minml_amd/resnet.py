@@ -44,9 +44,13 @@ def make_input(seed, batch, board, planes, p=0.3):
 
 
 class ResNet:
-    def __init__(self, context, batch, board, input_planes, channels, blocks, dtype, params_host, to_storage, chunk=None, fused=False):
-        """params_host: list from make_parameters; to_storage: fp32 ndarray -> ndarray in the storage type (identity or fp16 bits)."""
+    def __init__(self, context, batch, board, input_planes, channels, blocks, dtype, params_host, to_storage, chunk=None, fused=False,
+                 with_head=True):
+        """params_host: list from make_parameters; to_storage: fp32 ndarray -> ndarray in the storage type (identity or fp16 bits).
+        with_head=False leaves the 1x1 policy head out (params_host then ends with the last block convolution) and forward() returns
+        the trunk's activations [batch, board, board, channels]: the convolutional trunk of a larger network."""
         self.context = context
+        self.with_head = with_head
         self.fused = fused
         # True: also fuse across the residual blocks' boundaries (the block's result is written and transformed for the next block in one
         # launch). Identical results and less memory traffic, but measured 0.3 % to 1 % slower on MI355X than two launches there, whose
@@ -67,7 +71,10 @@ class ResNet:
         shape = (cb, board, board, channels)
         for _ in range(2 * blocks):
             self.layers.append(Conv2D(context, shape, channels, 3, "relu", True, self.dtype))
-        self.layers.append(Conv2D(context, shape, 1, 1, "linear", True, self.dtype))
+        if with_head:
+            self.layers.append(Conv2D(context, shape, 1, 1, "linear", True, self.dtype))
+        if len(params_host) != len(self.layers):
+            raise ValueError("expected parameters of %d layers, got %d" % (len(self.layers), len(params_host)))
         for layer, (w, b) in zip(self.layers, params_host):
             layer.setWeights(to_storage(w), to_storage(b))
 
@@ -76,7 +83,16 @@ class ResNet:
         # three rotating activation buffers per chunk: block input, intermediate, block output
         self.act = [ml.Tensor((cb, board, board, channels), self.dtype, context.device_index) for _ in range(3)]
         self.input = ml.Tensor((batch, board, board, input_planes), self.dtype, context.device_index)
-        self.output = ml.Tensor((batch, board, board, 1), self.dtype, context.device_index)
+        # without a head the trunk's activations of every sub-batch are collected here
+        self.output = ml.Tensor((batch, board, board, 1 if with_head else channels), self.dtype, context.device_index)
+
+    def _finish(self, a, start, n, ws):
+        """Head (or, without one, the copy of the trunk's result) of one sub-batch into its slice of the output."""
+        out = self._view_batch(self.output, start, n)
+        if self.with_head:
+            self.layers[-1].forward([a], out, ws)
+        else:
+            out.copyFrom(self.context, a)
 
     def setInput(self, x_storage):
         self.input.copyFromHost(self.context, x_storage)
@@ -112,7 +128,7 @@ class ResNet:
                 self._observe(2 + 2 * blk, c)
                 a, c = c, a
             ml.set_timer_label("head")
-            self.layers[-1].forward([a], self._view_batch(self.output, start, n), self.workspace)
+            self._finish(a, start, n, self.workspace)
             ml.set_timer_label(None)
         return self.output
 
@@ -157,8 +173,15 @@ class ResNet:
                         L[3 + 2 * blk].winograd_input(c, ws)
                 a, c = c, a
             ml.set_timer_label("head")
-            L[-1].forward([a], self._view_batch(self.output, start, n), ws)
+            self._finish(a, start, n, ws)
             ml.set_timer_label(None)
+        if self.fuse_layers:
+            # the whole-layer launch hands out producer / consumer roles among workgroups that must all be resident at once (64 per XCD);
+            # on a device shared with other work its bounded waits can give up, and the results are then invalid: ask, and say so
+            gave_up = ml.winogradLayerErrors(self.context)
+            if gave_up:
+                raise RuntimeError("%d workgroups of whole-layer Winograd launches gave up waiting for one another: the pass is invalid "
+                                   "(device shared with other work?); run with fuse_layers = False" % gave_up)
         return self.output
 
     def trunk_output(self):

@@ -39,11 +39,16 @@ class CpuResNet:
         shape = x.shape[:3] + (w.shape[0],)
         return e.winograd_output_transform(m, shape, b, add, act)
 
-    def forward(self, x, return_trunk=False):
+    def forward(self, x, return_trunk=False, per_layer=None):
+        """per_layer (a list) receives the output of every 3x3 layer in order (stem, then two per block)."""
         a = self._conv3x3(0, x, None, O.RELU)
+        if per_layer is not None:
+            per_layer.append(a)
         for blk in range(self.blocks):
             t = self._conv3x3(1 + 2 * blk, a, None, O.RELU)
             a = self._conv3x3(2 + 2 * blk, t, a, O.RELU)
+            if per_layer is not None:
+                per_layer.extend([t, a])
         w, b = self.params[-1]
         rows = a.shape[0] * a.shape[1] * a.shape[2]
         am = a.reshape(rows, a.shape[3])
@@ -90,3 +95,38 @@ class CpuQuantizedResNet:
             if per_layer is not None:
                 per_layer.extend([t, a])
         return self._conv(len(self.layers) - 1, a, None, O.LINEAR, O.FLOAT32)
+
+
+class CpuHybridNet:
+    """CPU execution of the hybrid network's layers that have a CPU implementation in the reference: the residual trunk (as CpuResNet,
+    without its head), then attention half-blocks (RMS normalisation -> dense qkv -> multi-head attention with the relative-position
+    table -> dense output with the residual as the product's C operand), then the 1x1 head. `params` has the layout of
+    minml_amd.hybridnet.make_hybrid_parameters, already in the storage type. per_layer (a dict) receives every intermediate tensor."""
+
+    def __init__(self, params_storage, blocks, heads):
+        self.params = params_storage
+        self.blocks = blocks
+        self.heads = heads
+        self.trunk = CpuResNet(params_storage["trunk"] + [params_storage["head"]], blocks, "oracle")
+
+    def attention_block(self, x, p, per_layer=None, index=0):
+        b, h, w, c = x.shape
+        rows = b * h * w
+        normed = O.rmsnorm_forward(x, p["gamma"])
+        qkv = O.gemm(normed.reshape(rows, c), p["w_qkv"], bias=p["b_qkv"], act=O.LINEAR).reshape(b, h, w, 3 * c)
+        att = O.multi_head_attention_forward(qkv, self.heads, p["table"], False)
+        out = O.gemm(att.reshape(rows, c), p["w_out"], beta=1.0, C=x.reshape(rows, c), bias=p["b_out"], act=O.LINEAR).reshape(b, h, w, c)
+        if per_layer is not None:
+            per_layer.update({"rmsnorm%d" % index: normed, "qkv%d" % index: qkv, "attention%d" % index: att, "block%d" % index: out})
+        return out
+
+    def forward(self, x, per_layer=None):
+        _, a = self.trunk.forward(x, return_trunk=True)
+        if per_layer is not None:
+            per_layer["trunk"] = a
+        for index, p in enumerate(self.params["attention"]):
+            a = self.attention_block(a, p, per_layer, index)
+        w, b = self.params["head"]
+        rows = a.shape[0] * a.shape[1] * a.shape[2]
+        head = O.gemm(a.reshape(rows, a.shape[3]), w.reshape(w.shape[0], -1), bias=b, act=O.LINEAR)
+        return head.reshape(a.shape[:3] + (w.shape[0],))

@@ -239,6 +239,32 @@ def test_convolution_linearity_at_full_size(ctx):
     assert np.array_equal(outs[0][100:101], sample)
 
 
+@pytest.mark.parametrize("channels,k", [(384, 3), (384, 5), (256, 5), (384, 1)])
+def test_config4_full_size_fp16(ctx, channels, k):
+    """Config 4 at its full size (B = 512, 19x19 boards, fp16, bias + residual + ReLU) at the widest channel counts: positions are
+    independent (a 2-position launch reproduces its slice of the full launch bit for bit: every output's reduction runs over K in the
+    same order whatever the number of rows), and a sample of positions matches the oracle's explicit convolution within 1e-2."""
+    rng = np.random.default_rng(46 + channels + k)
+    b = 512
+    x = random_tensor(rng, (b, 19, 19, channels), "float16")
+    wt = random_tensor(rng, (channels, k, k, channels), "float16", (2.0 / (k * k * channels)) ** 0.5)
+    bias = random_tensor(rng, (channels,), "float16", 0.01)
+    add = random_tensor(rng, (b, 19, 19, channels), "float16")
+    dx, dw, db, da = (ml.toDevice(ctx, a) for a in (x, wt, bias, add))
+    dy = ml.Tensor((b, 19, 19, channels), "float16")
+    ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, db, da, "relu")
+    got = dy.copyToHost(ctx)
+    per = 19 * 19 * channels
+    for first in (0, 301, 510):
+        part = ml.Tensor((2, 19, 19, channels), "float16")
+        ml.convolutionImplicitGemmForward(ctx, dx.view((2, 19, 19, channels), first * per), dw, part, db, da.view((2, 19, 19, channels), first * per), "relu")
+        assert mismatches(part.copyToHost(ctx), got[first:first + 2]) == 0
+    O.set_num_threads(8)
+    sample = [0, 255, 511]
+    want = O.conv2d_forward(x[sample], wt, bias, add[sample], O.RELU)
+    assert max_abs_rel(got[sample], want) <= 1e-2
+
+
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_elementwise_neighbours(ctx, dtype):
     rng = np.random.default_rng(7)

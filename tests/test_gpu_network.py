@@ -47,6 +47,32 @@ def test_config2_topology_fp16(ctx):
     assert max_abs_rel(head, want_head) <= 1e-2
 
 
+@pytest.mark.parametrize("config", [("config 1", 4, 128, 10, "float32", 0), ("config 2", 2, 256, 20, "float16", 1)])
+def test_error_per_layer_along_the_network(ctx, config):
+    """The benchmark networks at a batch the oracle finishes: the output of EVERY 3x3 layer (errors accumulated along the network, as a
+    user sees them) and the head against the CPU execution, and the figures printed so that the margin to the tolerance is on record."""
+    name, batch, channels, blocks, dtype, seed = config
+    O.set_num_threads(8)
+    conv = O.to_half if dtype == "float16" else (lambda a: np.ascontiguousarray(a, np.float32))
+    params = make_parameters(seed, 32, channels, blocks)
+    x = conv(make_input(seed, batch, 15, 32))
+    net = ResNet(ctx, batch, 15, 32, channels, blocks, dtype, params, conv)
+    seen = {}
+    net.observer = lambda index, tensor: seen.__setitem__(index, tensor.copyToHost(ctx))
+    net.setInput(x)
+    head = net.forward(fused=False).copyToHost(ctx)
+    want_layers = []
+    want_head = CpuResNet([(conv(w), conv(b)) for (w, b) in params], blocks, "oracle").forward(x, per_layer=want_layers)
+    errors = [max_abs_rel(seen[i], want_layers[i]) for i in range(len(want_layers))]
+    head_error = max_abs_rel(head, want_head)
+    print("%s topology, batch %d, %s: max-abs relative error per 3x3 layer: first %.2e, worst %.2e (layer %d), last %.2e; head %.2e; tolerance %.0e"
+          % (name, batch, dtype, errors[0], max(errors), int(np.argmax(errors)), errors[-1], head_error, TOL[dtype]), flush=True)
+    assert len(errors) == 1 + 2 * blocks
+    assert max(errors) <= TOL[dtype] and head_error <= TOL[dtype]
+    # the fused pass (output transform + next input transform in one launch) is bit-identical to the layer-by-layer pass
+    assert mismatches(net.forward(fused=True).copyToHost(ctx), head) == 0
+
+
 def test_per_layer_fp16(ctx):
     """Every layer of a 3-block fp16 network against the oracle run on the GPU's own input of that layer (no error accumulation)."""
     rng = np.random.default_rng(2)
