@@ -43,6 +43,8 @@ CONFIGS = {
     "cfg1_resnet10x128_fp32_b256": (256, 15, 32, 128, 10, "float32", 0),
     # the int8 form of configuration 2: same parameters (seed 1), per-channel int8 weights, per-tensor int8 activations calibrated on 64 batches
     "cfg3_resnet20x256_int8_b1024": (1024, 15, 32, 256, 20, "int8", 1),
+    # the part of configuration 5 that has a CPU reference: 10-block x 256 trunk, then 4 attention half-blocks (8 heads), N(0, 0.02) weights
+    "cfg5_hybrid10x256_attention4_fp16_b256": (256, 15, 32, 256, 10, "hybrid", 4),
 }
 PEAK_INT8_TOPS = 5000.0
 
@@ -159,6 +161,86 @@ def run_int8(args, ml):
     print(json.dumps(result))
 
 
+def run_hybrid(args, ml):
+    """Configuration 5 without its mixture-of-experts halves (those have no CPU implementation in the reference): residual trunk, four
+    attention half-blocks (RMS normalisation, dense qkv, attention with the relative-position table, dense output + residual), 1x1 head."""
+    import oracle as O
+    from oracle.cpu_net import CpuHybridNet
+    from minml_amd.hybridnet import HybridNet, make_hybrid_parameters
+    from minml_amd.resnet import make_input
+
+    batch, board, planes, channels, blocks, _, seed = CONFIGS[args.config]
+    attention_blocks, heads = 4, 8
+    to_storage = to_storage_factory("float16")
+    params = make_hybrid_parameters(seed, planes, channels, blocks, attention_blocks, heads, board)
+    x = make_input(seed, batch, board, planes)
+    ctx = ml.Context(0)
+    net = HybridNet(ctx, batch, board, planes, channels, blocks, heads, "float16", params, to_storage)
+    net.setInput(to_storage(x))
+    for _ in range(args.warmup):
+        net.forward()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        net.forward()
+    ctx.synchronize()
+    elapsed = time.perf_counter() - t0
+    timer = ml.KernelTimer(ctx)
+    ml.set_kernel_timer(timer)
+    for _ in range(max(1, min(args.steps, 5))):
+        net.forward()
+    kernels = timer.summary()
+    ml.set_kernel_timer(None)
+    per_pass = max(1, min(args.steps, 5))
+    breakdown = {name: {"launches_per_pass": n / per_pass, "avg_launch_us": t * 1e6, "ms_per_pass": n * t * 1e3 / per_pass}
+                 for name, (n, t) in sorted(kernels.items()) if "@" not in name}
+    tiles = batch * ((board + 3) // 4) ** 2
+    n_gemm, t_gemm = kernels.get("gemm_batched_v2", (0, float("nan")))
+    gemm_bytes = 2 * 36 * (2 * tiles * channels + channels * channels)
+    gemm_flops = 2.0 * 36 * tiles * channels * channels
+    n_att, t_att = kernels.get("multi_head_attention_forward", (0, float("nan")))
+    tokens = board * board
+    result = {
+        "metric": "positions/sec (%s)" % args.config, "value": batch / (elapsed / args.steps), "unit": "positions/sec", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": 1e3 * elapsed / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic (Bernoulli(0.3) input planes, N(0, 0.02) weights and position tables, N(0, 0.01) biases, seed %d)" % seed,
+        "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
+                   "attention_blocks": attention_blocks, "heads": heads, "mixture_of_experts_halves": "not included (no CPU reference)"},
+        "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
+        "roofline": {"bound": "hbm", "achieved": gemm_bytes / t_gemm / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": gemm_bytes / t_gemm / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                     "kernel": "kernel_gemm_stream_wide_nt (36 batched Winograd GEMMs of the trunk, M=%d N=K=%d)" % (tiles, channels),
+                     "algorithmic_bytes": gemm_bytes, "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6},
+        "gemm_mfma": {"achieved": gemm_flops / t_gemm / 1e12, "peak": PEAK_MFMA_TFLOPS["float16"], "unit": "TFLOP/s",
+                      "frac": gemm_flops / t_gemm / 1e12 / PEAK_MFMA_TFLOPS["float16"]},
+        "attention": {"avg_launch_us": t_att * 1e6, "launches_timed": n_att,
+                      "tflops": 4.0 * batch * heads * tokens * tokens * (channels // heads) / t_att / 1e12},
+        "entry_points": breakdown,
+    }
+    if args.cpu_seconds > 0:
+        cores = min(16, os.cpu_count() or 1)
+        O.set_num_threads(cores)
+        conv = to_storage
+        ps = {"trunk": [(conv(w), conv(b)) for (w, b) in params["trunk"]], "attention": [{k: conv(v) for k, v in blk.items()} for blk in params["attention"]],
+              "head": (conv(params["head"][0]), conv(params["head"][1]))}
+        cpu = CpuHybridNet(ps, blocks, heads)
+        xs = conv(x)
+        positions = 2
+        t0 = time.perf_counter()
+        cpu.forward(xs[:positions])
+        t = time.perf_counter() - t0
+        target = int(max(2, min(batch, args.cpu_seconds / max(t / positions, 1e-9))))
+        if target > positions:
+            positions = target
+            t0 = time.perf_counter()
+            cpu.forward(xs[:positions])
+            t = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": positions / t, "unit": "positions/sec", "cores": cores, "kind": "port",
+                                  "sample": "%d positions of the same network and inputs, one forward pass, %.1f s" % (positions, t)}
+    print(json.dumps(result))
+
+
 def copy_calibration(ml, ctx):
     """One copy kernel of known size (256 MiB read, 256 MiB written) so that a counter run can be scaled against it."""
     n = 128 * 1024 * 1024
@@ -196,6 +278,8 @@ def main():
 
     if CONFIGS[args.config][5] == "int8":
         return run_int8(args, ml)
+    if CONFIGS[args.config][5] == "hybrid":
+        return run_hybrid(args, ml)
     batch, board, planes, channels, blocks, dtype, seed = CONFIGS[args.config]
     chunk = args.chunk or DEFAULT_CHUNK.get(dtype, batch)
     to_storage = to_storage_factory(dtype)
