@@ -131,6 +131,18 @@ extern "C"
 			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
 			mlTensor_t next_matrices);
 	int hip_winograd_layer_errors(mlContext_t context);
+	/*
+	 * hip_winograd_layer_forward_static: hip_winograd_layer_forward with identical arguments and results that allocates nothing, neither
+	 * on the first call nor later. No counterpart in the reference; it is for callers that cannot allocate device memory: code under
+	 * HIP graph capture, serving loops and harnesses that forbid hipMalloc. hip_winograd_layer_forward keeps the counters and the
+	 * product scratch of its one-launch form in the context's growable workspace (hipMalloc on first use); this entry point keeps them in
+	 * a static device array of the library (18.1 MiB per GPU, held until the process ends) and clears its counters with a kernel. Limit:
+	 * at most 4096 images per call (larger batches are rejected with std::logic_error: split them). All calls on one GPU share that
+	 * array: calls that overlap on one GPU (two contexts, two threads) race; calls on one context run in stream order and are safe.
+	 */
+	void hip_winograd_layer_forward_static(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
+			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
+			mlTensor_t next_matrices);
 
 	/* ---- GEMMs (reference: cuda_backend.h:147-154; semantics of src/backend/cpu/gemm/gemm.cpp:34-83).
 	 *      C.dtype == INT32 selects the int8 x int8 -> int32 product (src/backend/cuda/gemms.cpp:119-130). ---- */

@@ -84,6 +84,7 @@ SIGNATURES = {
     "winograd_output_transform": (None, [_vp, _i, _T, _T, _T, _T, _i]),
     "winograd_output_input_transform": (None, [_vp, _i, _T, _T, _T, _S, _vp, _i, _T]),
     "winograd_layer_forward": (None, [_vp, _i, _T, _T, _T, _T, _T, _S, _vp, _i, _T]),
+    "winograd_layer_forward_static": (None, [_vp, _i, _T, _T, _T, _T, _T, _S, _vp, _i, _T]),
     "winograd_layer_errors": (_i, [_vp]),
     "gemm_v2": (None, [_vp, _c, _c, _f, _T, _T, _f, _T]),
     "gemm_batched_v2": (None, [_vp, _c, _c, _f, _T, _T, _f, _T]),

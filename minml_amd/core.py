@@ -343,10 +343,12 @@ def winogradOutputInputTransform(context, weight_shape, matrices, output_shape, 
             act_of(act), next_matrices.desc())
 
 
-def winogradLayerForward(context, weight_shape, input_matrices, weight_matrices, output_matrices, output_shape, output, bias, add, act, next_matrices):
+def winogradLayerForward(context, weight_shape, input_matrices, weight_matrices, output_matrices, output_shape, output, bias, add, act, next_matrices,
+                         static_memory=False):
     """Batched product, output transform and the next 3x3 layer's input transform in one call (no counterpart in the reference's
     math.hpp): identical to gemmBatched into `output_matrices` followed by winogradOutputInputTransform. For fp16, 256 channels and 16
-    tiles per image the product stays in the L2 cache and `output_matrices` is not touched."""
+    tiles per image the product stays in the L2 cache and `output_matrices` is not touched. static_memory=True calls the entry point
+    that allocates nothing (counters and scratch in the library's static device array; at most 4096 images per call)."""
     tile = get_winograd_tile(weight_shape, input_matrices.shape)
     _require_winograd_supported(tile, weight_shape[1], input_matrices.dtype)
     _require(_same_dtype(input_matrices, weight_matrices, output_matrices, next_matrices, output, bias, add), "dtype mismatch")
@@ -358,7 +360,8 @@ def winogradLayerForward(context, weight_shape, input_matrices, weight_matrices,
     _require(bias is None or bias.isEmpty() or bias.volume() == c, "bias must be [C]")
     _require(add is None or add.isEmpty() or add.shape == tuple(output_shape), "add must have the output's shape")
     _require(output is not None or c % 64 == 0, "without an output tensor the channel count must be a multiple of 64")
-    _launch("winograd_layer_forward", context.handle, tile, input_matrices.desc(), weight_matrices.desc(), output_matrices.desc(), _desc(bias), _desc(add),
+    _require(not static_memory or b <= 4096, "the static-memory form takes at most 4096 images per call")
+    _launch("winograd_layer_forward_static" if static_memory else "winograd_layer_forward", context.handle, tile, input_matrices.desc(), weight_matrices.desc(), output_matrices.desc(), _desc(bias), _desc(add),
             B.make_shape(output_shape), _ptr(output), act_of(act), next_matrices.desc())
 
 

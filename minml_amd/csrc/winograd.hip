@@ -1083,23 +1083,45 @@ namespace
 
 namespace
 {
-	/* device word that counts workgroups of the whole-layer kernel that gave up waiting; one per device, never freed */
-	unsigned int* layer_error_word()
+	/*
+	 * Device memory of the whole-layer launch that the library owns for the life of the process, one copy per device: the word that
+	 * counts workgroups which gave up waiting, the per-XCD counters and the product scratch (2 chunks of 36 x 64 x 256 halfs per XCD).
+	 * hip_winograd_layer_forward keeps counters and scratch in the context's growable workspace; hip_winograd_layer_forward_static, for
+	 * callers that must not allocate, keeps them here. The array's name is a host-side handle only: its device address is looked up
+	 * once per device with hipGetSymbolAddress and only that pointer is ever handed to kernels.
+	 */
+	constexpr size_t LAYER_ERROR_BYTES = 256;
+	constexpr size_t LAYER_SYNC_BYTES = sizeof(LayerSync) * LAYER_XCDS;
+	constexpr size_t LAYER_SCRATCH_BYTES = static_cast<size_t>(LAYER_XCDS) * LAYER_BUFFERS * LAYER_CHUNK_ELEMENTS * sizeof(half_t);
+	constexpr size_t LAYER_STATIC_BYTES = LAYER_ERROR_BYTES + (LAYER_SYNC_BYTES + 255) / 256 * 256 + LAYER_SCRATCH_BYTES; /* 18.1 MiB */
+	static __device__ __align__(256) uint8_t layer_static_memory[LAYER_STATIC_BYTES];
+
+	uint8_t* layer_static_pointer(int device_index)
 	{
 		static std::mutex guard;
-		static std::map<int, unsigned int*> words;
+		static std::map<int, uint8_t*> pointers;
 		std::lock_guard<std::mutex> lock(guard);
-		int device = 0;
-		MLHIP_CHECK(hipGetDevice(&device));
-		auto it = words.find(device);
-		if (it == words.end())
+		auto it = pointers.find(device_index);
+		if (it == pointers.end())
 		{
-			unsigned int *word = nullptr;
-			MLHIP_CHECK(hipMalloc(&word, sizeof(unsigned int)));
-			MLHIP_CHECK(hipMemset(word, 0, sizeof(unsigned int)));
-			it = words.insert(std::make_pair(device, word)).first;
+			MLHIP_CHECK(hipSetDevice(device_index)); /* every device holds its own copy of the array, at its own address */
+			void *address = nullptr;
+			MLHIP_CHECK(hipGetSymbolAddress(&address, HIP_SYMBOL(layer_static_memory)));
+			MLHIP_REQUIRE(address != nullptr, "Winograd layer: no device address for the library's static memory");
+			it = pointers.insert(std::make_pair(device_index, reinterpret_cast<uint8_t*>(address))).first;
 		}
 		return it->second;
+	}
+	/* device word that counts workgroups of the whole-layer kernel that gave up waiting (zero when the module is loaded) */
+	unsigned int* layer_error_word(int device_index)
+	{
+		return reinterpret_cast<unsigned int*>(layer_static_pointer(device_index));
+	}
+	/* clears `words` 32-bit words; a kernel rather than a memset node, so that callers may capture the launch sequence into a graph */
+	__global__ void kernel_clear_words(unsigned int *dst, unsigned int words)
+	{
+		for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
+			dst[i] = 0u;
 	}
 	bool layer_kernel_applies(const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlShape_t &shape, const mlTensor_t &bias,
 			const mlTensor_t &ext, const void *output, mlActivationType_t act)
@@ -1113,16 +1135,19 @@ namespace
 				&& device_compute_units() == 256;
 	}
 	void launch_layer(mlContext_t context, const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlTensor_t &bias, const mlTensor_t &ext,
-			const mlShape_t &shape, void *output, mlActivationType_t act, mlTensor_t &next)
+			const mlShape_t &shape, void *output, mlActivationType_t act, mlTensor_t &next, bool static_memory)
 	{
 		const hipStream_t stream = stream_of(context);
-		const size_t sync_bytes = sizeof(LayerSync) * LAYER_XCDS;
-		const size_t scratch_bytes = static_cast<size_t>(LAYER_XCDS) * LAYER_BUFFERS * LAYER_CHUNK_ELEMENTS * sizeof(half_t);
-		uint8_t *block = reinterpret_cast<uint8_t*>(get_workspace(context, sync_bytes + scratch_bytes));
+		const int device_index = get(context)->device_index;
+		const size_t sync_bytes = (LAYER_SYNC_BYTES + 255) / 256 * 256;
+		uint8_t *block = static_memory ? layer_static_pointer(device_index) + LAYER_ERROR_BYTES
+				: reinterpret_cast<uint8_t*>(get_workspace(context, sync_bytes + LAYER_SCRATCH_BYTES));
 		LayerSync *sync = reinterpret_cast<LayerSync*>(block);
 		half_t *scratch = reinterpret_cast<half_t*>(block + sync_bytes);
-		unsigned int *errors = layer_error_word();
-		MLHIP_CHECK(hipMemsetAsync(sync, 0, sync_bytes, stream));
+		unsigned int *errors = layer_error_word(device_index);
+		/* the counters start every launch at zero; the scratch needs no clearing (every row is written before it is read) */
+		hipLaunchKernelGGL(kernel_clear_words, dim3(32), dim3(256), 0, stream, reinterpret_cast<unsigned int*>(sync),
+				static_cast<unsigned int>(LAYER_SYNC_BYTES / sizeof(unsigned int)));
 		const int lds = 65536;
 		const dim3 grid(LAYER_XCDS * LAYER_WORKGROUPS_PER_XCD), block_dim(256);
 		const unsigned int spin_limit = 1u << 17; /* about a tenth of a second per wait before a workgroup gives up */
@@ -1260,9 +1285,9 @@ extern "C"
 		else
 			launch_output_input<float, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
 	}
-	void hip_winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
-			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
-			mlTensor_t next_matrices)
+	static void winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices,
+			mlTensor_t &output_matrices, const mlTensor_t &bias, const mlTensor_t &ext, const mlShape_t &output_shape, void *output, mlActivationType_t act,
+			mlTensor_t &next_matrices, bool static_memory)
 	{
 		MLHIP_REQUIRE(output_shape.rank == 4, "Winograd layer: output shape must be [B, H, W, C]");
 		require_supported(tile_size, input_matrices, input_matrices.dtype);
@@ -1283,9 +1308,12 @@ extern "C"
 		if (layer_kernel_applies(input_matrices, weight_matrices, output_shape, bias, ext, output, act))
 		{
 			mlTensor_t next = next_matrices;
-			launch_layer(context, input_matrices, weight_matrices, bias, ext, output_shape, output, act, next);
+			launch_layer(context, input_matrices, weight_matrices, bias, ext, output_shape, output, act, next, static_memory);
 			return;
 		}
+		if (static_memory)
+			MLHIP_REQUIRE(output_shape.dim[0] <= 4 * LAYER_XCDS * LAYER_MAX_CHUNKS,
+					"Winograd layer (static memory): at most 4096 images per call fit the library's static counters; split the batch");
 		/* every other shape: the batched product into the caller's matrices, then the fused (or two-step) transform */
 		MLHIP_REQUIRE(output_matrices.data != nullptr && output_matrices.dtype == input_matrices.dtype && output_matrices.rank == 3
 				&& output_matrices.dim[0] == 36 && static_cast<size_t>(output_matrices.dim[1]) == tiles && output_matrices.dim[2] == output_shape.dim[3],
@@ -1294,10 +1322,24 @@ extern "C"
 				shape_of(weight_matrices), weight_matrices.data, 'n', 't', 1.0f, 0.0f);
 		hip_winograd_output_input_transform(context, tile_size, output_matrices, bias, ext, output_shape, output, act, next_matrices);
 	}
+	void hip_winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
+			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
+			mlTensor_t next_matrices)
+	{
+		winograd_layer_forward(context, tile_size, input_matrices, weight_matrices, output_matrices, bias, ext, output_shape, output, act, next_matrices,
+				false);
+	}
+	void hip_winograd_layer_forward_static(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
+			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
+			mlTensor_t next_matrices)
+	{
+		winograd_layer_forward(context, tile_size, input_matrices, weight_matrices, output_matrices, bias, ext, output_shape, output, act, next_matrices,
+				true);
+	}
 	int hip_winograd_layer_errors(mlContext_t context)
 	{
 		MLHIP_CHECK(hipStreamSynchronize(stream_of(context)));
-		unsigned int *word = layer_error_word();
+		unsigned int *word = layer_error_word(get(context)->device_index);
 		unsigned int count = 0;
 		MLHIP_CHECK(hipMemcpy(&count, word, sizeof(count), hipMemcpyDeviceToHost));
 		if (count != 0)
