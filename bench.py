@@ -261,6 +261,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg2_resnet20x256_fp16_b1024", choices=sorted(CONFIGS))
     ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
+    ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments only; the metric is quoted at the default)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
     ap.add_argument("--unfused", action="store_true", help="run every layer as the reference's three calls (no cross-layer transform fusion)")
     ap.add_argument("--layer-launch", action="store_true", help="experimental: product and both transforms of a layer as one launch (slower)")
@@ -281,6 +282,7 @@ def main():
     if CONFIGS[args.config][5] == "hybrid":
         return run_hybrid(args, ml)
     batch, board, planes, channels, blocks, dtype, seed = CONFIGS[args.config]
+    batch = args.batch or batch
     chunk = args.chunk or DEFAULT_CHUNK.get(dtype, batch)
     to_storage = to_storage_factory(dtype)
     params = make_parameters(seed, planes, channels, blocks)

@@ -172,7 +172,13 @@ namespace
 			a_loader.c_bytes = static_cast<int>(c_bytes);
 			a_loader.fill = 0;
 			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(weights), filters_out, static_cast<int>(k_bytes) };
-			launch_gemm_dma<T>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, make_epilogue());
+			if constexpr (sizeof(T) == 2) /* the fp16 hot path gets its epilogue's common cases fixed at compile time */
+				specialise_epilogue(make_epilogue(), [&](const auto &ep)
+				{
+					launch_gemm_dma<T>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, ep);
+				});
+			else
+				launch_gemm_dma<T>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, make_epilogue());
 		}
 		else if (fast)
 		{

@@ -17,7 +17,15 @@ namespace mlhip
 	 * uninitialised). Activations other than LINEAR / RELU are applied to the value rounded to the storage type, because the reference
 	 * runs them as a second pass over the stored matrix (src/backend/cpu/gemm/gemm.cpp:81-82).
 	 */
-	template<typename T>
+	/*
+	 * Which parts of an epilogue are known when the kernel is compiled. A kernel whose epilogue decides activation / bias / residual at
+	 * run time carries the code of every activation and a branch per decision in its innermost store loop; with the common cases fixed
+	 * at compile time (ReLU or linear, bias present, residual present or not) that loop is straight-line code. EPILOGUE_RUNTIME keeps
+	 * the decision in the functor's fields; `specialise_epilogue` picks the compile-time form that matches them.
+	 */
+	constexpr int EPILOGUE_RUNTIME = -1;
+
+	template<typename T, int ACT = EPILOGUE_RUNTIME, int WITH_C = EPILOGUE_RUNTIME, int WITH_BIAS = EPILOGUE_RUNTIME>
 	struct FloatEpilogue
 	{
 			T *D;
@@ -30,15 +38,53 @@ namespace mlhip
 			bool vectorized; /* N % 4 == 0 and D, C, bias 4-element aligned */
 			static constexpr bool has_c = true;
 
+			__device__ __forceinline__ int activation() const
+			{
+				if constexpr (ACT == EPILOGUE_RUNTIME)
+					return act;
+				else
+					return ACT;
+			}
+			__device__ __forceinline__ bool with_c() const
+			{
+				if constexpr (WITH_C == EPILOGUE_RUNTIME)
+					return beta != 0.0f;
+				else
+					return WITH_C != 0;
+			}
+			__device__ __forceinline__ bool with_bias() const
+			{
+				if constexpr (WITH_BIAS == EPILOGUE_RUNTIME)
+					return bias != nullptr;
+				else
+					return WITH_BIAS != 0;
+			}
+			/* the same epilogue with other parts fixed at compile time (the caller guarantees that they agree with the fields) */
+			template<int A, int C, int B>
+			FloatEpilogue<T, A, C, B> fixed() const
+			{
+				FloatEpilogue<T, A, C, B> e;
+				e.D = D;
+				e.C = this->C;
+				e.bias = bias;
+				e.N = N;
+				e.row_stride = row_stride;
+				e.alpha = alpha;
+				e.beta = beta;
+				e.act = act;
+				e.vectorized = vectorized;
+				return e;
+			}
 			__device__ __forceinline__ float finish(float x) const
 			{
-				if (act == ACTIVATION_RELU)
+				const int a = activation();
+				if (a == ACTIVATION_RELU)
 					return fmaxf(x, 0.0f);
-				if (act != ACTIVATION_LINEAR)
+				if (a != ACTIVATION_LINEAR)
 				{
 					if constexpr (sizeof(T) == 2)
 						x = half_bits_to_float(half_bits_rtz(x));
-					return activate(act, x);
+					return activate(a, x);
 				}
 				return x;
 			}
@@ -57,14 +103,14 @@ namespace mlhip
 			};
 			__device__ __forceinline__ bool has_extra() const
 			{
-				return beta != 0.0f;
+				return with_c();
 			}
 			__device__ __forceinline__ Column load_column(int n) const
 			{
 				Column col;
 				Vec<T, 4> b;
 				b.zero();
-				if (bias != nullptr)
+				if (with_bias())
 					b.load(bias + n);
 #pragma unroll
 				for (int e = 0; e < 4; e++)
@@ -84,13 +130,13 @@ namespace mlhip
 #pragma unroll
 				for (int e = 0; e < 4; e++)
 					out.v[e] = acc[e] * alpha;
-				if (bias != nullptr)
+				if (with_bias())
 				{
 #pragma unroll
 					for (int e = 0; e < 4; e++)
 						out.v[e] += col.bias[e];
 				}
-				if (beta != 0.0f)
+				if (with_c())
 				{
 					float c[4];
 					if constexpr (sizeof(T) == 2)
@@ -126,7 +172,7 @@ namespace mlhip
 #pragma unroll
 					for (int e = 0; e < 4; e++)
 						out.v[e] = acc[e] * alpha;
-					if (bias != nullptr)
+					if (with_bias())
 					{
 						Vec<T, 4> b;
 						b.load(bias + n);
@@ -134,7 +180,7 @@ namespace mlhip
 						for (int e = 0; e < 4; e++)
 							out.v[e] += b.v[e];
 					}
-					if (beta != 0.0f)
+					if (with_c())
 					{
 						Vec<T, 4> c;
 						c.load(C + offset);
@@ -154,9 +200,9 @@ namespace mlhip
 						if (n + e < N)
 						{
 							float x = acc[e] * alpha;
-							if (bias != nullptr)
+							if (with_bias())
 								x += Storage<T>::load(bias + n + e);
-							if (beta != 0.0f)
+							if (with_c())
 								x += beta * Storage<T>::load(C + offset + e);
 							Storage<T>::store(D + offset + e, finish(x));
 						}
@@ -258,7 +304,7 @@ namespace mlhip
 		return static_cast<int>(q);
 	}
 
-	template<typename OutT> /* int8_t (requantised), float or half_t (dequantised) */
+	template<typename OutT, int ACT = EPILOGUE_RUNTIME, int WITH_EXT = EPILOGUE_RUNTIME> /* OutT: int8_t (requantised), float or half_t (dequantised) */
 	struct RequantEpilogue
 	{
 			OutT *D;
@@ -273,6 +319,38 @@ namespace mlhip
 			bool vectorized; /* N % 4 == 0 and all pointers 4-element aligned */
 			static constexpr bool has_c = false;
 
+			__device__ __forceinline__ int activation() const
+			{
+				if constexpr (ACT == EPILOGUE_RUNTIME)
+					return act;
+				else
+					return ACT;
+			}
+			__device__ __forceinline__ bool with_ext() const
+			{
+				if constexpr (WITH_EXT == EPILOGUE_RUNTIME)
+					return ext != nullptr;
+				else
+					return WITH_EXT != 0;
+			}
+			template<int A, int E>
+			RequantEpilogue<OutT, A, E> fixed() const
+			{
+				RequantEpilogue<OutT, A, E> e;
+				e.D = D;
+				e.scales = scales;
+				e.bias = bias;
+				e.ext = ext;
+				e.N = N;
+				e.row_stride = row_stride;
+				e.ext_scale = ext_scale;
+				e.ext_shift = ext_shift;
+				e.inv_scale = inv_scale;
+				e.inv_shift = inv_shift;
+				e.act = act;
+				e.vectorized = vectorized;
+				return e;
+			}
 			struct Column
 			{
 					float4_t scales, bias;
@@ -290,7 +368,7 @@ namespace mlhip
 			}
 			__device__ __forceinline__ bool has_extra() const
 			{
-				return ext != nullptr;
+				return with_ext();
 			}
 			__device__ __forceinline__ Extra load_extra(int m, int n) const
 			{
@@ -306,7 +384,7 @@ namespace mlhip
 				for (int e = 0; e < 4; e++)
 				{
 					const int ext_val = static_cast<int>(static_cast<int8_t>((x.packed >> (8 * e)) & 0xffu));
-					vals[e] = requant_value(acc[e], col.scales[e], col.bias[e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+					vals[e] = requant_value(acc[e], col.scales[e], col.bias[e], with_ext(), ext_val, ext_scale, ext_shift, activation());
 				}
 				if constexpr (sizeof(OutT) == 1)
 				{
@@ -336,13 +414,13 @@ namespace mlhip
 					const float4_t s = *reinterpret_cast<const float4_t*>(scales + n);
 					const float4_t b = *reinterpret_cast<const float4_t*>(bias + n);
 					uint32_t e_packed = 0;
-					if (ext != nullptr)
+					if (with_ext())
 						e_packed = *reinterpret_cast<const uint32_t*>(ext + offset);
 #pragma unroll
 					for (int e = 0; e < 4; e++)
 					{
 						const int ext_val = static_cast<int>(static_cast<int8_t>((e_packed >> (8 * e)) & 0xffu));
-						vals[e] = requant_value(acc[e], s[e], b[e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+						vals[e] = requant_value(acc[e], s[e], b[e], with_ext(), ext_val, ext_scale, ext_shift, activation());
 					}
 					if constexpr (sizeof(OutT) == 1)
 					{
@@ -367,8 +445,8 @@ namespace mlhip
 					for (int e = 0; e < 4; e++)
 						if (n + e < N)
 						{
-							const int ext_val = (ext != nullptr) ? static_cast<int>(ext[offset + e]) : 0;
-							const float v = requant_value(acc[e], scales[n + e], bias[n + e], ext != nullptr, ext_val, ext_scale, ext_shift, act);
+							const int ext_val = with_ext() ? static_cast<int>(ext[offset + e]) : 0;
+							const float v = requant_value(acc[e], scales[n + e], bias[n + e], with_ext(), ext_val, ext_scale, ext_shift, activation());
 							if constexpr (sizeof(OutT) == 1)
 								D[offset + e] = static_cast<OutT>(quantize_to_int8(v, inv_scale, inv_shift));
 							else
@@ -377,6 +455,54 @@ namespace mlhip
 				}
 			}
 	};
+
+	/*
+	 * Calls launch(e') with e' = `e` whose activation and optional inputs are compile-time constants where they are the hot path's
+	 * (ReLU or linear; bias present; residual present or not; 4-element groups whole and aligned), and with `e` itself otherwise.
+	 * `launch` is a generic lambda: every form it is called with is a kernel instantiation of its own.
+	 */
+	template<typename T, typename Launch>
+	inline void specialise_epilogue(const FloatEpilogue<T> &e, Launch &&launch)
+	{
+		const bool eligible = e.vectorized && e.bias != nullptr && (e.act == ACTIVATION_RELU || e.act == ACTIVATION_LINEAR);
+		if (!eligible)
+			launch(e);
+		else if (e.act == ACTIVATION_RELU)
+		{
+			if (e.beta != 0.0f)
+				launch(e.template fixed<ACTIVATION_RELU, 1, 1>());
+			else
+				launch(e.template fixed<ACTIVATION_RELU, 0, 1>());
+		}
+		else
+		{
+			if (e.beta != 0.0f)
+				launch(e.template fixed<ACTIVATION_LINEAR, 1, 1>());
+			else
+				launch(e.template fixed<ACTIVATION_LINEAR, 0, 1>());
+		}
+	}
+	template<typename OutT, typename Launch>
+	inline void specialise_epilogue(const RequantEpilogue<OutT> &e, Launch &&launch)
+	{
+		const bool eligible = e.vectorized && (e.act == ACTIVATION_RELU || e.act == ACTIVATION_LINEAR);
+		if (!eligible)
+			launch(e);
+		else if (e.act == ACTIVATION_RELU)
+		{
+			if (e.ext != nullptr)
+				launch(e.template fixed<ACTIVATION_RELU, 1>());
+			else
+				launch(e.template fixed<ACTIVATION_RELU, 0>());
+		}
+		else
+		{
+			if (e.ext != nullptr)
+				launch(e.template fixed<ACTIVATION_LINEAR, 1>());
+			else
+				launch(e.template fixed<ACTIVATION_LINEAR, 0>());
+		}
+	}
 } /* namespace mlhip */
 
 #endif /* MINML_AMD_EPILOGUES_HPP_ */

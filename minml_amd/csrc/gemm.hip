@@ -136,7 +136,10 @@ namespace mlhip
 			else if (g.dtype == DTYPE_FLOAT32 && plain)
 				launch_stream_gemm<float>(stream, sg, PlainStore { });
 			else if (g.dtype == DTYPE_FLOAT16 && vectorized)
-				launch_stream_gemm<half_t>(stream, sg, make_float_epilogue<half_t>(g, true));
+				specialise_epilogue(make_float_epilogue<half_t>(g, true), [&](const auto &ep)
+				{
+					launch_stream_gemm<half_t>(stream, sg, ep);
+				});
 			else if (g.dtype == DTYPE_FLOAT32 && vectorized)
 				launch_stream_gemm<float>(stream, sg, make_float_epilogue<float>(g, true));
 			else if (g.dtype == DTYPE_INT8 && vectorized && g.bias == nullptr && g.act == ACTIVATION_LINEAR)

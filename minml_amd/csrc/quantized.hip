@@ -175,7 +175,10 @@ namespace
 		if (fast && kernel_h == 1 && kernel_w == 1 && ep.vectorized && stream_gemm_applies(M, 1, k_bytes))
 		{ /* a 1x1 convolution with a short K row is bound by HBM: the persistent streaming kernel on the [B*H*W, Cin] view */
 			const StreamGemmArgs sg { input, weights, nullptr, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0 };
-			launch_stream_gemm<int8_t>(stream, sg, ep);
+			specialise_epilogue(ep, [&](const auto &fixed)
+			{
+				launch_stream_gemm<int8_t>(stream, sg, fixed);
+			});
 		}
 		else if (fast && filters_in % 128 == 0)
 		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */
@@ -189,7 +192,10 @@ namespace
 			a_loader.c_bytes = filters_in;
 			a_loader.fill = input_zero & 0xff; /* a 1x1 kernel never pads, so an out-of-range zero point is harmless there */
 			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(weights), filters_out, static_cast<int>(k_bytes) };
-			launch_gemm_dma<int8_t>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, ep);
+			specialise_epilogue(ep, [&](const auto &fixed)
+			{
+				launch_gemm_dma<int8_t>(stream, a_loader, b_loader, M, filters_out, static_cast<int>(k_bytes), 1, 0, 0, 0, fixed);
+			});
 		}
 		else if (fast)
 		{
