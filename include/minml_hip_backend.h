@@ -199,6 +199,23 @@ extern "C"
 			bool symmetric); /* input [B,H,W,(3 - symmetric) E] = q,k,v per token; weights = position table [heads, 2r-1, round_up(2r-1, 4)] or NULL;
 			                    bias and workspace unused; backward_data must be NULL */
 
+	/* ---- mixture of experts: the feed-forward half of the hybrid networks' transformer blocks (reference: cuda_backend.h:245-265,
+	 *      src/backend/cuda/kernels/moe.cu, callers src/layers/{Router,GatherTokens,MixtureOfExperts,ScatterTokens}.cpp). The reference
+	 *      implements these for its CUDA backend only (src/core/math.cpp:1328-1491 does nothing on the CPU). fp16 and fp32, inference only.
+	 *      x = router scores [B, H, W, E]; indices_and_values [B, 2, E, K] in the tensors' type: plane 0 = token index held by slot k of
+	 *      expert e (-1 = empty), plane 1 = its gate. Equal scores are ordered by ascending token index. ---- */
+	void hip_expert_choice_routing_forward(mlContext_t context, const mlTensor_t x,
+			mlTensor_t indices_and_values); /* every expert takes its K best tokens of each image, best first; gate = sigmoid(score) (moe.cu:438-479) */
+	void hip_token_choice_routing_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t bias,
+			mlTensor_t indices_and_values); /* every token takes the expert with the largest score + bias[E]; gate = its softmax; K best per expert (moe.cu:191-350) */
+	void hip_hash_routing(mlContext_t context, const mlTensor_t x, mlTensor_t indices_and_values); /* token k * E + e -> slot k of expert e, gate 1 (moe.cu:167-189) */
+	void hip_gather_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta,
+			mlTensor_t y); /* x [B, H, W, C] -> y [B, K, E, C] = x[token] + beta * y; empty slots: beta * y (0 when beta = 0) (moe.cu:505-532) */
+	void hip_moe_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, float beta, mlTensor_t y,
+			mlActivationType_t act); /* y [B, K, E, N] = act(x [B, K, E, C] . w[e] [N, C]^T + b [E, N] + beta * y), one dense layer per expert (moe.cu:1395-1432) */
+	void hip_scatter_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta,
+			mlTensor_t y); /* y [B, H, W, C] = beta * y + sum over the slots holding each token of gate * x [B, K, E, C], in fp32, experts ascending (moe.cu:559-582) */
+
 	/* ---- additions with no counterpart in the reference ABI ----
 	 * hip_quantized_conv_forward: the whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 (int8 implicit GEMM with
 	 * zero-point padding, int32 accumulation, per-channel scale + bias, optional int8 residual, activation, requantisation)

@@ -105,6 +105,12 @@ SIGNATURES = {
     "rmsnorm_forward": (None, [_vp, _S, _i, _vp, _vp, _vp]),
     "multi_head_attention_get_workspace_size": (_i, [_S, _S, _i, _b]),
     "multi_head_attention_forward": (None, [_vp, _S, _S, _S, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _b]),
+    "expert_choice_routing_forward": (None, [_vp, _T, _T]),
+    "token_choice_routing_forward": (None, [_vp, _T, _T, _T]),
+    "hash_routing": (None, [_vp, _T, _T]),
+    "gather_tokens_forward": (None, [_vp, _T, _T, _f, _T]),
+    "moe_forward": (None, [_vp, _T, _T, _T, _f, _T, _i]),
+    "scatter_tokens_forward": (None, [_vp, _T, _T, _f, _T]),
     "quantized_conv_forward": (None, [_vp, _S, _S, _vp, _Q, _vp, _vp, _vp, _i, _vp, _Q, _vp, _Q, _i]),
     "get_stream": (_vp, [_vp]),
 }

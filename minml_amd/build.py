@@ -16,7 +16,7 @@ LIB = os.path.join(HERE, "libminml_hip.so")
 # the backend library exports nothing but the backend's interface
 CEILINGS_LIB = os.path.join(HERE, "libminml_ceilings.so")
 
-SOURCES = ["runtime.hip", "winograd.hip", "gemm.hip", "conv.hip", "quantized.hip", "elementwise.hip", "heads.hip", "attention.hip", "cuda_stubs.cpp"]
+SOURCES = ["runtime.hip", "winograd.hip", "gemm.hip", "conv.hip", "quantized.hip", "elementwise.hip", "heads.hip", "attention.hip", "moe.hip", "cuda_stubs.cpp"]
 # packed fp32 VALU forms are switched off for all device code; the host pass does not know the feature and says so (harmless)
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

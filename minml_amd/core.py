@@ -568,6 +568,62 @@ def multiHeadAttentionForward(context, input, output, weights, bias, workspace, 
             num_heads, bool(symmetric))
 
 
+def _require_routing(input, indices_and_values):
+    _require(len(input.shape) == 4 and len(indices_and_values.shape) == 4 and indices_and_values.shape[1] == 2, "scores [B, H, W, E], routing table [B, 2, E, K]")
+    _require(input.shape[0] == indices_and_values.shape[0] and input.shape[3] == indices_and_values.shape[2], "batch size or number of experts differ")
+    _require(_same_dtype(input, indices_and_values) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "fp16 or fp32 tensors of one type")
+    _require(input.shape[1] * input.shape[2] <= 2048 and input.shape[3] <= 4096 and input.shape[0] <= 65535, "at most 2048 tokens per image, 4096 experts")
+
+
+def expertChoiceRoutingForward(context, input, indicesAndValues):
+    """Every expert takes its K best tokens of each image (reference: src/core/math.cpp:1371-1383)."""
+    _require_routing(input, indicesAndValues)
+    _launch("expert_choice_routing_forward", context.handle, input.desc(), indicesAndValues.desc())
+
+
+def tokenChoiceRoutingForward(context, input, bias, indicesAndValues):
+    """Every token takes the expert with the largest score + bias (reference: src/core/math.cpp:1343-1355)."""
+    _require_routing(input, indicesAndValues)
+    _require(bias is None or bias.isEmpty() or (bias.volume() == input.shape[3] and bias.dtype == input.dtype), "bias must be [E] of the scores' type")
+    _launch("token_choice_routing_forward", context.handle, input.desc(), _desc(bias), indicesAndValues.desc())
+
+
+def hashRouting(context, input, indicesAndValues):
+    """reference: src/core/math.cpp:1329-1341."""
+    _require_routing(input, indicesAndValues)
+    _launch("hash_routing", context.handle, input.desc(), indicesAndValues.desc())
+
+
+def gatherTokensForward(context, input, indicesAndValues, beta, output):
+    """[B, H, W, C] -> [B, K, E, C] (reference: src/core/math.cpp:1410-1422)."""
+    _require(len(input.shape) == 4 and len(output.shape) == 4 and len(indicesAndValues.shape) == 4 and indicesAndValues.shape[1] == 2, "rank-4 tensors")
+    b, k, e, c = output.shape
+    _require(input.shape[0] == b and input.shape[3] == c and indicesAndValues.shape == (b, 2, e, k), "shapes do not agree")
+    _require(_same_dtype(input, output, indicesAndValues) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "fp16 or fp32 tensors of one type")
+    _launch("gather_tokens_forward", context.handle, input.desc(), indicesAndValues.desc(), beta, output.desc())
+
+
+def moeForward(context, input, weights, bias, beta, output, act):
+    """One dense layer per expert on [B, K, E, C] (reference: src/core/math.cpp:1462-1475)."""
+    _require(len(input.shape) == 4 and len(output.shape) == 4 and len(weights.shape) == 3, "x [B, K, E, C], weights [E, N, C], y [B, K, E, N]")
+    b, k, e, c = input.shape
+    n = weights.shape[1]
+    _require(weights.shape == (e, n, c) and output.shape == (b, k, e, n), "shapes do not agree")
+    _require(bias is None or bias.isEmpty() or bias.volume() == e * n, "bias must be [E, N]")
+    _require(_same_dtype(input, output, weights, bias) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "fp16 or fp32 tensors of one type")
+    _require(b * k <= 0x7fffffff and e <= 65535, "too large")
+    _launch("moe_forward", context.handle, input.desc(), weights.desc(), _desc(bias), beta, output.desc(), act_of(act))
+
+
+def scatterTokensForward(context, input, indicesAndValues, beta, output):
+    """[B, K, E, C] -> [B, H, W, C], every token the gated sum of its slots (reference: src/core/math.cpp:1436-1448)."""
+    _require(len(input.shape) == 4 and len(output.shape) == 4 and len(indicesAndValues.shape) == 4 and indicesAndValues.shape[1] == 2, "rank-4 tensors")
+    b, k, e, c = input.shape
+    _require(output.shape[0] == b and output.shape[3] == c and indicesAndValues.shape == (b, 2, e, k), "shapes do not agree")
+    _require(_same_dtype(input, output, indicesAndValues) and input.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "fp16 or fp32 tensors of one type")
+    _launch("scatter_tokens_forward", context.handle, input.desc(), indicesAndValues.desc(), beta, output.desc())
+
+
 def foldBatchnorm(context, layer_weights, layer_bias, bn_weights, bn_bias, bn_avg_var):
     """Folds a batch normalisation into the preceding layer's weights and bias, in place (reference: src/core/math.cpp:786-802, which
     also synchronises with the context afterwards)."""

@@ -61,17 +61,11 @@ MLHIP_STUB(cuda_rmsnorm_backward)
 /* attention, mixture of experts */
 MLHIP_STUB(cuda_multi_head_attention_backward)
 MLHIP_STUB(cuda_group_gemm)
-MLHIP_STUB(cuda_hash_routing)
-MLHIP_STUB(cuda_token_choice_routing_forward)
 MLHIP_STUB(cuda_token_choice_routing_backward)
-MLHIP_STUB(cuda_expert_choice_routing_forward)
 MLHIP_STUB(cuda_expert_choice_routing_backward)
 MLHIP_STUB(cuda_select_top_k)
-MLHIP_STUB(cuda_gather_tokens_forward)
 MLHIP_STUB(cuda_gather_tokens_backward)
-MLHIP_STUB(cuda_scatter_tokens_forward)
 MLHIP_STUB(cuda_scatter_tokens_backward)
-MLHIP_STUB(cuda_moe_forward)
 MLHIP_STUB(cuda_moe_backward)
 /* backward passes, softmax, tensor helpers */
 MLHIP_STUB(cuda_activation_backward)

@@ -36,6 +36,7 @@ namespace mlhip
 			float alpha, beta;
 			int act;
 			bool vectorized; /* N % 4 == 0 and D, C, bias 4-element aligned */
+			int bias_batch_stride = 0; /* elements between the biases of consecutive matrices of a batch (0: one bias for all) */
 			static constexpr bool has_c = true;
 
 			__device__ __forceinline__ int activation() const
@@ -73,6 +74,7 @@ namespace mlhip
 				e.beta = beta;
 				e.act = act;
 				e.vectorized = vectorized;
+				e.bias_batch_stride = bias_batch_stride;
 				return e;
 			}
 			__device__ __forceinline__ float finish(float x) const

@@ -100,6 +100,7 @@ namespace mlhip
 			const uint8_t *base;
 			int rows;
 			int k_bytes;
+			int row_stride_bytes = 0; /* bytes between consecutive rows; 0 = rows are contiguous (k_bytes apart) */
 
 			struct Row
 			{
@@ -111,7 +112,7 @@ namespace mlhip
 			};
 			__device__ __forceinline__ Row begin_row(int row) const
 			{
-				return Row { base + static_cast<size_t>(min(row, rows - 1)) * k_bytes };
+				return Row { base + static_cast<size_t>(min(row, rows - 1)) * (row_stride_bytes != 0 ? row_stride_bytes : k_bytes) };
 			}
 			__device__ __forceinline__ Step first_step() const
 			{
@@ -288,37 +289,55 @@ namespace mlhip
 			const bool n_valid = n < epilogue.N;
 			const int n_safe = n_valid ? n : 0;
 			const typename Epilogue::Column column = epilogue.load_column(n_safe);
-			typename Epilogue::Extra extra[2][PASSES];
-			auto request_extras = [&](auto block, auto buffer)
+			/*
+			 * A wavefront whose whole sub-tile lies inside the matrix (all but the last row / column tiles) runs the UNCHECKED form:
+			 * no per-pass range test, hence no branch between the side-input loads and their use, so the compiler counts the
+			 * outstanding loads exactly instead of draining them all (vmcnt(0)) in front of every pass.
+			 */
+			const bool inside = __builtin_amdgcn_readfirstlane(
+					static_cast<int>(m0 + wave_m * Cfg::WM + Cfg::WM <= M && n0 + wave_n * Cfg::WN + Cfg::WN <= epilogue.N)) != 0;
+			auto run = [&](auto checked_tag)
 			{
-				constexpr int i = decltype(block)::value, buf = decltype(buffer)::value;
-				if (!epilogue.has_extra())
-					return;
-#pragma unroll
-				for (int pass = 0; pass < PASSES; pass++)
-					extra[buf][pass] = epilogue.load_extra(min(m_base + 32 * i + pass * ROWS_PER_PASS, M - 1), n_safe);
-			};
-			request_extras(std::integral_constant<int, 0>(), std::integral_constant<int, 0>());
-			static_for<Cfg::BLOCKS_M>([&](auto block)
-			{
-				constexpr int i = decltype(block)::value;
-				fill_slab(block);
-				if constexpr (i + 1 < Cfg::BLOCKS_M)
-					request_extras(std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>());
-#pragma unroll
-				for (int pass = 0; pass < PASSES; pass++)
+				constexpr bool CHECKED = decltype(checked_tag)::value;
+				typename Epilogue::Extra extra[2][PASSES];
+				auto request_extras = [&](auto block, auto buffer)
 				{
-					const int row = pass * ROWS_PER_PASS + row_in_pass;
-					const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + col);
-					const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
-					if (m < M && n_valid)
+					constexpr int i = decltype(block)::value, buf = decltype(buffer)::value;
+					if (!epilogue.has_extra())
+						return;
+#pragma unroll
+					for (int pass = 0; pass < PASSES; pass++)
 					{
-						acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
-						epilogue.apply(m, n, vals, column, extra[i & 1][pass]);
+						const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
+						extra[buf][pass] = epilogue.load_extra(CHECKED ? min(m, M - 1) : m, n_safe);
 					}
-				}
-				release_slab();
-			});
+				};
+				request_extras(std::integral_constant<int, 0>(), std::integral_constant<int, 0>());
+				static_for<Cfg::BLOCKS_M>([&](auto block)
+				{
+					constexpr int i = decltype(block)::value;
+					fill_slab(block);
+					if constexpr (i + 1 < Cfg::BLOCKS_M)
+						request_extras(std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>());
+#pragma unroll
+					for (int pass = 0; pass < PASSES; pass++)
+					{
+						const int row = pass * ROWS_PER_PASS + row_in_pass;
+						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + col);
+						const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
+						if (!CHECKED || (m < M && n_valid))
+						{
+							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
+							epilogue.apply(m, n, vals, column, extra[i & 1][pass]);
+						}
+					}
+					release_slab();
+				});
+			};
+			if (inside)
+				run(std::false_type());
+			else
+				run(std::true_type());
 		}
 		else
 		{
@@ -540,7 +559,11 @@ namespace mlhip
 		b_loader.base += batch * stride_b_bytes;
 		epilogue.D += batch * stride_c;
 		if constexpr (Epilogue::has_c)
+		{
 			epilogue.C += batch * stride_c;
+			if (epilogue.bias != nullptr)
+				epilogue.bias += batch * epilogue.bias_batch_stride; /* 0 unless every matrix of the batch has its own bias */
+		}
 		gemm_tile_dma<T, Cfg>(a_loader, b_loader, M, k_bytes, tile_m * Cfg::BM, tile_n * Cfg::BN, lds, epilogue);
 	}
 

@@ -1,0 +1,538 @@
+/*
+ * moe.hip — mixture-of-experts steps of the hybrid networks' feed-forward blocks: routing (expert choice, token choice, hash),
+ * gathering the routed tokens per expert, the per-expert dense layers, and scattering the experts' results back to their tokens.
+ *
+ * Interface and tensor layouts follow the reference's device backend (declarations: include/minml/backend/cuda_backend.h:245-265;
+ * kernels: src/backend/cuda/kernels/moe.cu; callers: src/layers/{Router,GatherTokens,MixtureOfExperts,ScatterTokens}.cpp). The reference
+ * has no CPU implementation of these operations (src/core/math.cpp:1328-1491), so their arithmetic is fixed here where its kernels
+ * leave it open: equal scores are ordered by ascending token index (the reference: by its sorting network), and the scatter sums a
+ * token's contributions in fp32 in ascending expert order and rounds once (the reference: atomic additions in the storage type).
+ *
+ *   scores                 [B, H, W, E]      one router logit per token and expert
+ *   indices_and_values     [B, 2, E, K]      storage type; plane 0 = token index of slot k of expert e (as a number, -1 = empty), plane 1 = gate
+ *   gathered tokens        [B, K, E, C]
+ *   expert weights / bias  [E, N, C] / [E, N]
+ */
+#include "common.hpp"
+#include "device_utils.hpp"
+#include "epilogues.hpp"
+#include "gemm_dma.hpp"
+
+namespace
+{
+	using namespace mlhip;
+
+	constexpr int MAX_ROUTED_TOKENS = 2048; /* tokens per image that the in-LDS sorts take */
+
+	__device__ __forceinline__ uint32_t ascending_bits(float v)
+	{
+		const uint32_t u = __builtin_bit_cast(uint32_t, v);
+		return u ^ ((u >> 31) ? 0xffffffffu : 0x80000000u);
+	}
+	__device__ __forceinline__ float from_ascending_bits(uint32_t s)
+	{
+		const uint32_t u = s ^ ((s >> 31) ? 0x80000000u : 0xffffffffu);
+		return __builtin_bit_cast(float, u);
+	}
+	/* in-place bitonic sort of `count` (a power of two) 64-bit keys in LDS, ascending; all threads of the workgroup take part */
+	__device__ __forceinline__ void sort_keys(uint64_t *keys, int count)
+	{
+		for (int k = 2; k <= count; k <<= 1)
+			for (int j = k >> 1; j > 0; j >>= 1)
+			{
+				for (int i = threadIdx.x; i < count; i += blockDim.x)
+				{
+					const int partner = i ^ j;
+					if (partner > i)
+					{
+						const bool ascending = ((i & k) == 0);
+						const uint64_t a = keys[i], b = keys[partner];
+						if ((a > b) == ascending)
+						{
+							keys[i] = b;
+							keys[partner] = a;
+						}
+					}
+				}
+				__syncthreads();
+			}
+	}
+	__device__ __forceinline__ int next_power_of_two(int n)
+	{
+		int p = 1;
+		while (p < n)
+			p <<= 1;
+		return p;
+	}
+
+	/* one workgroup per (expert, image): the expert's `capacity` best tokens, best first, gate = sigmoid(score) */
+	template<typename T>
+	__global__ __launch_bounds__(256) void kernel_expert_choice_routing(const T *scores, T *indices_and_values, int tokens, int experts, int capacity)
+	{
+		__shared__ uint64_t keys[MAX_ROUTED_TOKENS];
+		const int e = blockIdx.x, b = blockIdx.y;
+		const int padded = next_power_of_two(tokens);
+		for (int t = threadIdx.x; t < padded; t += blockDim.x)
+		{
+			uint64_t key = ~0ull;
+			if (t < tokens)
+			{
+				const float s = Storage<T>::load(scores + (static_cast<size_t>(b) * tokens + t) * experts + e);
+				key = (static_cast<uint64_t>(~ascending_bits(s)) << 32) | static_cast<uint32_t>(t); /* score descending, then token ascending */
+			}
+			keys[t] = key;
+		}
+		__syncthreads();
+		sort_keys(keys, padded);
+		T *index_row = indices_and_values + ((static_cast<size_t>(b) * 2 + 0) * experts + e) * capacity;
+		T *value_row = indices_and_values + ((static_cast<size_t>(b) * 2 + 1) * experts + e) * capacity;
+		for (int k = threadIdx.x; k < capacity; k += blockDim.x)
+		{
+			if (k < tokens)
+			{
+				const uint64_t key = keys[k];
+				const float s = from_ascending_bits(~static_cast<uint32_t>(key >> 32));
+				Storage<T>::store(index_row + k, static_cast<float>(static_cast<uint32_t>(key)));
+				Storage<T>::store(value_row + k, 1.0f / (1.0f + expf(-s)));
+			}
+			else
+			{
+				Storage<T>::store(index_row + k, -1.0f);
+				Storage<T>::store(value_row + k, 0.0f);
+			}
+		}
+	}
+
+	/*
+	 * One workgroup per image. Every token takes the expert with the largest score + bias (the lowest index among equals); its gate is
+	 * softmax(scores)[that expert] with the maximum of score + bias as the shift, kept in the storage type; the tokens are then sorted
+	 * by (expert, gate descending, token) and every expert keeps the first `capacity` of its run.
+	 */
+	template<typename T>
+	__global__ __launch_bounds__(256) void kernel_token_choice_routing(const T *scores, const T *bias, T *indices_and_values, int tokens, int experts,
+			int capacity)
+	{
+		__shared__ uint64_t keys[MAX_ROUTED_TOKENS];
+		__shared__ int first[4096 + 1]; /* first[e] = position of expert e's run in the sorted keys, -1 if it has none; count in last[e] */
+		__shared__ int last[4096 + 1];
+		const int b = blockIdx.x;
+		const int padded = next_power_of_two(tokens);
+		for (int e = threadIdx.x; e < experts; e += blockDim.x)
+		{
+			first[e] = -1;
+			last[e] = -1;
+		}
+		for (int t = threadIdx.x; t < padded; t += blockDim.x)
+		{
+			uint64_t key = ~0ull;
+			if (t < tokens)
+			{
+				const T *row = scores + (static_cast<size_t>(b) * tokens + t) * experts;
+				float best = 0.0f;
+				int choice = 0;
+				for (int e = 0; e < experts; e++)
+				{
+					const float plus = Storage<T>::load(row + e) + ((bias != nullptr) ? Storage<T>::load(bias + e) : 0.0f);
+					if (e == 0 || plus > best)
+					{
+						best = plus;
+						choice = e;
+					}
+				}
+				float total = 0.0f;
+				for (int e = 0; e < experts; e++)
+					total = total + expf(Storage<T>::load(row + e) - best);
+				float gate = expf(Storage<T>::load(row + choice) - best) / total;
+				if constexpr (sizeof(T) == 2)
+					gate = half_bits_to_float(half_bits_rtz(gate));
+				key = (static_cast<uint64_t>(choice) << 52) | (static_cast<uint64_t>(~ascending_bits(gate)) << 20) | static_cast<uint64_t>(t);
+			}
+			keys[t] = key;
+		}
+		__syncthreads();
+		sort_keys(keys, padded);
+		for (int p = threadIdx.x; p < tokens; p += blockDim.x)
+		{
+			const int e = static_cast<int>(keys[p] >> 52);
+			if (p == 0 || static_cast<int>(keys[p - 1] >> 52) != e)
+				first[e] = p;
+			if (p + 1 == tokens || static_cast<int>(keys[p + 1] >> 52) != e)
+				last[e] = p;
+		}
+		__syncthreads();
+		for (int i = threadIdx.x; i < experts * capacity; i += blockDim.x)
+		{
+			const int e = i / capacity, k = i - e * capacity;
+			T *index_slot = indices_and_values + ((static_cast<size_t>(b) * 2 + 0) * experts + e) * capacity + k;
+			T *value_slot = indices_and_values + ((static_cast<size_t>(b) * 2 + 1) * experts + e) * capacity + k;
+			if (first[e] >= 0 && first[e] + k <= last[e])
+			{
+				const uint64_t key = keys[first[e] + k];
+				Storage<T>::store(index_slot, static_cast<float>(static_cast<uint32_t>(key & 0xfffffu)));
+				Storage<T>::store(value_slot, from_ascending_bits(~static_cast<uint32_t>(key >> 20)));
+			}
+			else
+			{
+				Storage<T>::store(index_slot, -1.0f);
+				Storage<T>::store(value_slot, 0.0f);
+			}
+		}
+	}
+
+	template<typename T>
+	__global__ __launch_bounds__(256) void kernel_hash_routing(T *indices_and_values, int batch, int tokens, int experts, int capacity)
+	{
+		const size_t total = static_cast<size_t>(batch) * experts * capacity;
+		for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += static_cast<size_t>(gridDim.x) * blockDim.x)
+		{
+			const int k = static_cast<int>(i % capacity);
+			const int e = static_cast<int>((i / capacity) % experts);
+			const size_t b = i / (static_cast<size_t>(capacity) * experts);
+			const int token = k * experts + e;
+			const bool filled = token < tokens;
+			Storage<T>::store(indices_and_values + ((b * 2 + 0) * experts + e) * capacity + k, filled ? static_cast<float>(token) : -1.0f);
+			Storage<T>::store(indices_and_values + ((b * 2 + 1) * experts + e) * capacity + k, filled ? 1.0f : 0.0f);
+		}
+	}
+
+	/* one thread per group of VEC channels of one gathered row (b, k, e) */
+	template<typename T, int VEC>
+	__global__ __launch_bounds__(256) void kernel_gather_tokens(const T *x, const T *indices_and_values, T *y, float beta, size_t groups, int tokens, int channels,
+			int experts, int capacity)
+	{
+		const int per_row = channels / VEC;
+		for (size_t g = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; g < groups; g += static_cast<size_t>(gridDim.x) * blockDim.x)
+		{
+			const size_t row = g / per_row; /* (b * K + k) * E + e */
+			const int c = static_cast<int>(g - row * per_row) * VEC;
+			const int e = static_cast<int>(row % experts);
+			const size_t bk = row / experts;
+			const int k = static_cast<int>(bk % capacity);
+			const size_t b = bk / capacity;
+			const int token = static_cast<int>(Storage<T>::load(indices_and_values + ((b * 2 + 0) * experts + e) * capacity + k));
+			Vec<T, VEC> out;
+			out.zero();
+			if (beta != 0.0f)
+			{
+				out.load(y + row * channels + c);
+#pragma unroll
+				for (int i = 0; i < VEC; i++)
+					out.v[i] *= beta;
+			}
+			if (token >= 0)
+			{
+				Vec<T, VEC> in;
+				in.load(x + (b * tokens + token) * channels + c);
+#pragma unroll
+				for (int i = 0; i < VEC; i++)
+					out.v[i] = in.v[i] + out.v[i];
+			}
+			out.store(y + row * channels + c);
+		}
+	}
+
+	/*
+	 * One wavefront per token and block of 64 * VEC channels: the slots that hold the token are found by scanning the image's index
+	 * table expert by expert (a token occupies at most one slot per expert), and their gated rows are summed in fp32 in that order.
+	 */
+	template<typename T, int VEC>
+	__global__ __launch_bounds__(256) void kernel_scatter_tokens(const T *x, const T *indices_and_values, T *y, float beta, size_t total_tokens, int tokens,
+			int channels, int experts, int capacity)
+	{
+#pragma clang fp contract(off)
+		const int lane = threadIdx.x & 63;
+		const size_t slot = static_cast<size_t>(blockIdx.x) * (blockDim.x >> 6) + (threadIdx.x >> 6);
+		const int channel_blocks = (channels + 64 * VEC - 1) / (64 * VEC);
+		const size_t global_token = slot / channel_blocks;
+		if (global_token >= total_tokens)
+			return;
+		const int c = (static_cast<int>(slot % channel_blocks) * 64 + lane) * VEC;
+		const size_t b = global_token / tokens;
+		const int token = static_cast<int>(global_token - b * tokens);
+		const bool active = c < channels;
+		Vec<T, VEC> acc;
+		acc.zero();
+		if (beta != 0.0f && active)
+		{
+			acc.load(y + global_token * channels + c);
+#pragma unroll
+			for (int i = 0; i < VEC; i++)
+				acc.v[i] *= beta;
+		}
+		for (int e = 0; e < experts; e++)
+		{
+			const T *index_row = indices_and_values + ((b * 2 + 0) * experts + e) * capacity;
+			for (int k0 = 0; k0 < capacity; k0 += 64)
+			{
+				const int k = k0 + lane;
+				const bool match = (k < capacity) && (static_cast<int>(Storage<T>::load(index_row + k)) == token);
+				const unsigned long long hits = __ballot(match);
+				if (hits != 0ull)
+				{
+					const int found = k0 + __builtin_ctzll(hits);
+					const float gate = Storage<T>::load(indices_and_values + ((b * 2 + 1) * experts + e) * capacity + found);
+					if (active)
+					{
+						Vec<T, VEC> in;
+						in.load(x + ((b * capacity + found) * experts + e) * channels + c);
+#pragma unroll
+						for (int i = 0; i < VEC; i++)
+						{
+							const float scaled = gate * in.v[i];
+							acc.v[i] = acc.v[i] + scaled;
+						}
+					}
+					break; /* at most one slot per expert */
+				}
+			}
+		}
+		if (active)
+			acc.store(y + global_token * channels + c);
+	}
+
+	/* fallback of the expert layers for shapes the tile engine does not take: one thread per output element */
+	template<typename T>
+	__global__ __launch_bounds__(256) void kernel_moe_generic(const T *x, const T *w, const T *bias, T *y, float beta, size_t outputs, int experts, int neurons,
+			int channels, int act)
+	{
+		for (size_t o = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; o < outputs; o += static_cast<size_t>(gridDim.x) * blockDim.x)
+		{
+			const int n = static_cast<int>(o % neurons);
+			const size_t row = o / neurons; /* (b * K + k) * E + e */
+			const int e = static_cast<int>(row % experts);
+			const T *a = x + row * channels;
+			const T *wr = w + (static_cast<size_t>(e) * neurons + n) * channels;
+			float acc = 0.0f;
+			for (int c = 0; c < channels; c++)
+				acc = fmaf(Storage<T>::load(a + c), Storage<T>::load(wr + c), acc);
+			if (bias != nullptr)
+				acc += Storage<T>::load(bias + static_cast<size_t>(e) * neurons + n);
+			if (beta != 0.0f)
+				acc += beta * Storage<T>::load(y + o);
+			if (act == ACTIVATION_RELU)
+				acc = fmaxf(acc, 0.0f);
+			else if (act != ACTIVATION_LINEAR)
+			{
+				if constexpr (sizeof(T) == 2)
+					acc = half_bits_to_float(half_bits_rtz(acc));
+				acc = activate(act, acc);
+			}
+			Storage<T>::store(y + o, acc);
+		}
+	}
+
+	unsigned int grid_for(size_t items)
+	{
+		const size_t blocks = (items + 255) / 256;
+		return static_cast<unsigned int>(blocks < 65536 * 16 ? (blocks > 0 ? blocks : 1) : 65536 * 16);
+	}
+	void require_routing_tensors(const mlTensor_t &x, const mlTensor_t &iv, const char *what)
+	{
+		MLHIP_REQUIRE(x.rank == 4 && iv.rank == 4 && iv.dim[1] == 2, std::string(what) + ": scores must be [B, H, W, E] and the routing table [B, 2, E, K]");
+		MLHIP_REQUIRE(x.dim[0] == iv.dim[0] && x.dim[3] == iv.dim[2], std::string(what) + ": batch size or number of experts differ");
+		MLHIP_REQUIRE(x.dtype == iv.dtype && (x.dtype == DTYPE_FLOAT16 || x.dtype == DTYPE_FLOAT32), std::string(what) + ": fp16 or fp32 tensors of one type");
+		MLHIP_REQUIRE(x.dim[1] * x.dim[2] <= MAX_ROUTED_TOKENS, std::string(what) + ": at most 2048 tokens per image");
+		MLHIP_REQUIRE(iv.dim[2] <= 4096 && x.dim[1] * x.dim[2] < (1 << 20), std::string(what) + ": too many experts");
+	}
+	template<typename T>
+	bool vector_ok(int channels, int vec, const void *a, const void *b)
+	{
+		const size_t bytes = sizeof(T) * vec;
+		return channels % vec == 0 && reinterpret_cast<uintptr_t>(a) % bytes == 0 && reinterpret_cast<uintptr_t>(b) % bytes == 0;
+	}
+}
+
+extern "C"
+{
+	using namespace mlhip;
+
+	void hip_expert_choice_routing_forward(mlContext_t context, const mlTensor_t x, mlTensor_t indices_and_values)
+	{
+		require_routing_tensors(x, indices_and_values, "expert_choice_routing_forward");
+		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
+		if (batch == 0 || experts == 0 || capacity == 0)
+			return;
+		MLHIP_REQUIRE(x.data != nullptr && indices_and_values.data != nullptr && batch <= 65535, "expert_choice_routing_forward: null tensor or batch above 65535");
+		const dim3 grid(experts, batch);
+		if (x.dtype == DTYPE_FLOAT16)
+			hipLaunchKernelGGL(kernel_expert_choice_routing<half_t>, grid, dim3(256), 0, stream_of(context), ptr<const half_t>(x), ptr<half_t>(indices_and_values),
+					tokens, experts, capacity);
+		else
+			hipLaunchKernelGGL(kernel_expert_choice_routing<float>, grid, dim3(256), 0, stream_of(context), ptr<const float>(x), ptr<float>(indices_and_values),
+					tokens, experts, capacity);
+		MLHIP_CHECK(hipGetLastError());
+	}
+	void hip_token_choice_routing_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t bias, mlTensor_t indices_and_values)
+	{
+		require_routing_tensors(x, indices_and_values, "token_choice_routing_forward");
+		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
+		if (batch == 0 || experts == 0 || capacity == 0)
+			return;
+		if (bias.data != nullptr)
+			MLHIP_REQUIRE(bias.dtype == x.dtype && volume(bias) == static_cast<size_t>(experts), "token_choice_routing_forward: bias must be [E] of the scores' type");
+		MLHIP_REQUIRE(x.data != nullptr && indices_and_values.data != nullptr, "token_choice_routing_forward: null tensor");
+		if (x.dtype == DTYPE_FLOAT16)
+			hipLaunchKernelGGL(kernel_token_choice_routing<half_t>, dim3(batch), dim3(256), 0, stream_of(context), ptr<const half_t>(x), ptr<const half_t>(bias),
+					ptr<half_t>(indices_and_values), tokens, experts, capacity);
+		else
+			hipLaunchKernelGGL(kernel_token_choice_routing<float>, dim3(batch), dim3(256), 0, stream_of(context), ptr<const float>(x), ptr<const float>(bias),
+					ptr<float>(indices_and_values), tokens, experts, capacity);
+		MLHIP_CHECK(hipGetLastError());
+	}
+	void hip_hash_routing(mlContext_t context, const mlTensor_t x, mlTensor_t indices_and_values)
+	{
+		require_routing_tensors(x, indices_and_values, "hash_routing");
+		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
+		const size_t total = static_cast<size_t>(batch) * experts * capacity;
+		if (total == 0)
+			return;
+		MLHIP_REQUIRE(indices_and_values.data != nullptr, "hash_routing: null tensor");
+		if (x.dtype == DTYPE_FLOAT16)
+			hipLaunchKernelGGL(kernel_hash_routing<half_t>, dim3(grid_for(total)), dim3(256), 0, stream_of(context), ptr<half_t>(indices_and_values), batch, tokens,
+					experts, capacity);
+		else
+			hipLaunchKernelGGL(kernel_hash_routing<float>, dim3(grid_for(total)), dim3(256), 0, stream_of(context), ptr<float>(indices_and_values), batch, tokens,
+					experts, capacity);
+		MLHIP_CHECK(hipGetLastError());
+	}
+
+	void hip_gather_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta, mlTensor_t y)
+	{
+		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && indices_and_values.rank == 4 && indices_and_values.dim[1] == 2,
+				"gather_tokens_forward: x [B, H, W, C], routing table [B, 2, E, K], y [B, K, E, C]");
+		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], channels = x.dim[3], capacity = y.dim[1], experts = y.dim[2];
+		MLHIP_REQUIRE(y.dim[0] == batch && y.dim[3] == channels && indices_and_values.dim[0] == batch && indices_and_values.dim[2] == experts
+				&& indices_and_values.dim[3] == capacity, "gather_tokens_forward: shapes do not agree");
+		MLHIP_REQUIRE(x.dtype == y.dtype && x.dtype == indices_and_values.dtype && (x.dtype == DTYPE_FLOAT16 || x.dtype == DTYPE_FLOAT32),
+				"gather_tokens_forward: fp16 or fp32 tensors of one type");
+		const size_t rows = static_cast<size_t>(batch) * capacity * experts;
+		if (rows == 0 || channels == 0)
+			return;
+		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && indices_and_values.data != nullptr, "gather_tokens_forward: null tensor");
+		const hipStream_t stream = stream_of(context);
+#define MLHIP_GATHER(T, VEC) hipLaunchKernelGGL((kernel_gather_tokens<T, VEC>), dim3(grid_for(rows * (channels / VEC))), dim3(256), 0, stream, ptr<const T>(x), \
+		ptr<const T>(indices_and_values), ptr<T>(y), beta, rows * (channels / VEC), tokens, channels, experts, capacity)
+		if (x.dtype == DTYPE_FLOAT16)
+		{
+			if (vector_ok<half_t>(channels, 8, x.data, y.data))
+				MLHIP_GATHER(half_t, 8);
+			else
+				MLHIP_GATHER(half_t, 1);
+		}
+		else
+		{
+			if (vector_ok<float>(channels, 4, x.data, y.data))
+				MLHIP_GATHER(float, 4);
+			else
+				MLHIP_GATHER(float, 1);
+		}
+#undef MLHIP_GATHER
+		MLHIP_CHECK(hipGetLastError());
+	}
+	void hip_scatter_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta, mlTensor_t y)
+	{
+		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && indices_and_values.rank == 4 && indices_and_values.dim[1] == 2,
+				"scatter_tokens_forward: x [B, K, E, C], routing table [B, 2, E, K], y [B, H, W, C]");
+		const int batch = y.dim[0], tokens = y.dim[1] * y.dim[2], channels = y.dim[3], capacity = x.dim[1], experts = x.dim[2];
+		MLHIP_REQUIRE(x.dim[0] == batch && x.dim[3] == channels && indices_and_values.dim[0] == batch && indices_and_values.dim[2] == experts
+				&& indices_and_values.dim[3] == capacity, "scatter_tokens_forward: shapes do not agree");
+		MLHIP_REQUIRE(x.dtype == y.dtype && x.dtype == indices_and_values.dtype && (x.dtype == DTYPE_FLOAT16 || x.dtype == DTYPE_FLOAT32),
+				"scatter_tokens_forward: fp16 or fp32 tensors of one type");
+		const size_t total_tokens = static_cast<size_t>(batch) * tokens;
+		if (total_tokens == 0 || channels == 0)
+			return;
+		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && indices_and_values.data != nullptr, "scatter_tokens_forward: null tensor");
+		const hipStream_t stream = stream_of(context);
+#define MLHIP_SCATTER(T, VEC) \
+		do { \
+			const size_t wavefronts = total_tokens * ((channels + 64 * VEC - 1) / (64 * VEC)); \
+			MLHIP_REQUIRE((wavefronts + 3) / 4 <= 0x7fffffffu, "scatter_tokens_forward: tensor too large for one launch"); \
+			hipLaunchKernelGGL((kernel_scatter_tokens<T, VEC>), dim3(static_cast<unsigned int>((wavefronts + 3) / 4)), dim3(256), 0, stream, ptr<const T>(x), \
+					ptr<const T>(indices_and_values), ptr<T>(y), beta, total_tokens, tokens, channels, experts, capacity); \
+		} while (0)
+		if (x.dtype == DTYPE_FLOAT16)
+		{
+			if (vector_ok<half_t>(channels, 4, x.data, y.data))
+				MLHIP_SCATTER(half_t, 4);
+			else
+				MLHIP_SCATTER(half_t, 1);
+		}
+		else
+		{
+			if (vector_ok<float>(channels, 4, x.data, y.data))
+				MLHIP_SCATTER(float, 4);
+			else
+				MLHIP_SCATTER(float, 1);
+		}
+#undef MLHIP_SCATTER
+		MLHIP_CHECK(hipGetLastError());
+	}
+
+	void hip_moe_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, float beta, mlTensor_t y, mlActivationType_t act)
+	{
+		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && w.rank == 3, "moe_forward: x [B, K, E, C], weights [E, N, C], y [B, K, E, N]");
+		const int batch = x.dim[0], capacity = x.dim[1], experts = x.dim[2], channels = x.dim[3], neurons = w.dim[1];
+		MLHIP_REQUIRE(w.dim[0] == experts && w.dim[2] == channels && y.dim[0] == batch && y.dim[1] == capacity && y.dim[2] == experts && y.dim[3] == neurons,
+				"moe_forward: shapes do not agree");
+		MLHIP_REQUIRE(x.dtype == y.dtype && x.dtype == w.dtype && (x.dtype == DTYPE_FLOAT16 || x.dtype == DTYPE_FLOAT32),
+				"moe_forward: fp16 or fp32 tensors of one type");
+		if (b.data != nullptr)
+			MLHIP_REQUIRE(b.dtype == x.dtype && volume(b) == static_cast<size_t>(experts) * neurons, "moe_forward: bias must be [E, N] of the tensors' type");
+		const size_t rows = static_cast<size_t>(batch) * capacity;
+		if (rows == 0 || experts == 0 || neurons == 0)
+			return;
+		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && w.data != nullptr && rows <= 0x7fffffffu && experts <= 65535, "moe_forward: null tensor or too large");
+		const hipStream_t stream = stream_of(context);
+		const int esize = size_of(x.dtype);
+		const size_t k_bytes = static_cast<size_t>(channels) * esize;
+		const auto aligned = [](const void *p, size_t a) { return reinterpret_cast<uintptr_t>(p) % a == 0; };
+		const bool vectorized = neurons % 4 == 0 && aligned(y.data, 4 * esize) && aligned(b.data, 4 * esize);
+		const bool dma = channels > 0 && k_bytes % 128 == 0 && aligned(x.data, 16) && aligned(w.data, 16) && static_cast<size_t>(experts) * k_bytes <= 0x7fffffffu;
+		if (dma)
+		{
+			/* expert e multiplies the rows (b, k) of x, which lie E * C elements apart, by its own [N, C] weights into rows E * N apart */
+			DenseDmaRows a_loader { reinterpret_cast<const uint8_t*>(x.data), static_cast<int>(rows), static_cast<int>(k_bytes) };
+			a_loader.row_stride_bytes = static_cast<int>(static_cast<size_t>(experts) * k_bytes);
+			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(w.data), neurons, static_cast<int>(k_bytes) };
+			const auto launch = [&](auto zero)
+			{
+				typedef decltype(zero) T;
+				FloatEpilogue<T> ep;
+				ep.D = reinterpret_cast<T*>(y.data);
+				ep.C = reinterpret_cast<const T*>(y.data);
+				ep.bias = reinterpret_cast<const T*>(b.data);
+				ep.N = neurons;
+				ep.row_stride = experts * neurons;
+				ep.alpha = 1.0f;
+				ep.beta = beta;
+				ep.act = act;
+				ep.vectorized = vectorized;
+				ep.bias_batch_stride = neurons;
+				launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
+						static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), ep);
+			};
+			if (x.dtype == DTYPE_FLOAT16)
+				launch(half_t(0));
+			else
+				launch(0.0f);
+		}
+		else
+		{
+			const size_t outputs = rows * experts * neurons;
+			if (x.dtype == DTYPE_FLOAT16)
+				hipLaunchKernelGGL(kernel_moe_generic<half_t>, dim3(grid_for(outputs)), dim3(256), 0, stream, ptr<const half_t>(x), ptr<const half_t>(w),
+						ptr<const half_t>(b), ptr<half_t>(y), beta, outputs, experts, neurons, channels, static_cast<int>(act));
+			else
+				hipLaunchKernelGGL(kernel_moe_generic<float>, dim3(grid_for(outputs)), dim3(256), 0, stream, ptr<const float>(x), ptr<const float>(w),
+						ptr<const float>(b), ptr<float>(y), beta, outputs, experts, neurons, channels, static_cast<int>(act));
+		}
+		MLHIP_CHECK(hipGetLastError());
+	}
+} /* extern "C" */
+
+MLHIP_ALSO_AS_CUDA(expert_choice_routing_forward)
+MLHIP_ALSO_AS_CUDA(token_choice_routing_forward)
+MLHIP_ALSO_AS_CUDA(hash_routing)
+MLHIP_ALSO_AS_CUDA(gather_tokens_forward)
+MLHIP_ALSO_AS_CUDA(scatter_tokens_forward)
+MLHIP_ALSO_AS_CUDA(moe_forward)
