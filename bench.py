@@ -45,6 +45,9 @@ CONFIGS = {
     "cfg3_resnet20x256_int8_b1024": (1024, 15, 32, 256, 20, "int8", 1),
     # the part of configuration 5 that has a CPU reference: 10-block x 256 trunk, then 4 attention half-blocks (8 heads), N(0, 0.02) weights
     "cfg5_hybrid10x256_attention4_fp16_b256": (256, 15, 32, 256, 10, "hybrid", 4),
+    # the whole of configuration 5: the same plus the feed-forward halves as mixtures of 8 experts (hidden 1024, expert-choice routing
+    # with capacity factor 2 = two experts per token on average); that half has no CPU reference (checked against this repository's own CPU statement)
+    "cfg5_hybrid10x256_attention4_moe8_fp16_b256": (256, 15, 32, 256, 10, "hybrid_moe", 4),
 }
 PEAK_INT8_TOPS = 5000.0
 
@@ -169,13 +172,14 @@ def run_hybrid(args, ml):
     from minml_amd.hybridnet import HybridNet, make_hybrid_parameters
     from minml_amd.resnet import make_input
 
-    batch, board, planes, channels, blocks, _, seed = CONFIGS[args.config]
+    batch, board, planes, channels, blocks, kind, seed = CONFIGS[args.config]
+    moe = kind == "hybrid_moe"
     attention_blocks, heads = 4, 8
     to_storage = to_storage_factory("float16")
     params = make_hybrid_parameters(seed, planes, channels, blocks, attention_blocks, heads, board)
     x = make_input(seed, batch, board, planes)
     ctx = ml.Context(0)
-    net = HybridNet(ctx, batch, board, planes, channels, blocks, heads, "float16", params, to_storage)
+    net = HybridNet(ctx, batch, board, planes, channels, blocks, heads, "float16", params, to_storage, moe=moe)
     net.setInput(to_storage(x))
     for _ in range(args.warmup):
         net.forward()
@@ -206,7 +210,8 @@ def run_hybrid(args, ml):
         "vs_baseline": None, "dtype": "f16",
         "data": "synthetic (Bernoulli(0.3) input planes, N(0, 0.02) weights and position tables, N(0, 0.01) biases, seed %d)" % seed,
         "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
-                   "attention_blocks": attention_blocks, "heads": heads, "mixture_of_experts_halves": "not included (no CPU reference)"},
+                   "attention_blocks": attention_blocks, "heads": heads,
+                   "mixture_of_experts_halves": "8 experts, hidden 1024, expert-choice routing, capacity factor 2" if moe else "not included (no CPU reference)"},
         "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
         "roofline": {"bound": "hbm", "achieved": gemm_bytes / t_gemm / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": gemm_bytes / t_gemm / 1e9 / PEAK_HBM_GBS, "traffic": None,
@@ -224,17 +229,23 @@ def run_hybrid(args, ml):
         conv = to_storage
         ps = {"trunk": [(conv(w), conv(b)) for (w, b) in params["trunk"]], "attention": [{k: conv(v) for k, v in blk.items()} for blk in params["attention"]],
               "head": (conv(params["head"][0]), conv(params["head"][1]))}
+        capacity = None
+        if moe:
+            from minml_amd.hybridnet import get_capacity
+
+            ps["ffn"] = [{k: conv(v) for k, v in blk.items()} for blk in params["ffn"]]
+            capacity = get_capacity(2.0, board * board, 8)
         cpu = CpuHybridNet(ps, blocks, heads)
         xs = conv(x)
         positions = 2
         t0 = time.perf_counter()
-        cpu.forward(xs[:positions])
+        cpu.forward(xs[:positions], moe_capacity=capacity)
         t = time.perf_counter() - t0
         target = int(max(2, min(batch, args.cpu_seconds / max(t / positions, 1e-9))))
         if target > positions:
             positions = target
             t0 = time.perf_counter()
-            cpu.forward(xs[:positions])
+            cpu.forward(xs[:positions], moe_capacity=capacity)
             t = time.perf_counter() - t0
         result["cpu_baseline"] = {"value": positions / t, "unit": "positions/sec", "cores": cores, "kind": "port",
                                   "sample": "%d positions of the same network and inputs, one forward pass, %.1f s" % (positions, t)}
@@ -279,7 +290,7 @@ def main():
 
     if CONFIGS[args.config][5] == "int8":
         return run_int8(args, ml)
-    if CONFIGS[args.config][5] == "hybrid":
+    if CONFIGS[args.config][5] in ("hybrid", "hybrid_moe"):
         return run_hybrid(args, ml)
     batch, board, planes, channels, blocks, dtype, seed = CONFIGS[args.config]
     batch = args.batch or batch

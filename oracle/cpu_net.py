@@ -120,12 +120,38 @@ class CpuHybridNet:
             per_layer.update({"rmsnorm%d" % index: normed, "qkv%d" % index: qkv, "attention%d" % index: att, "block%d" % index: out})
         return out
 
-    def forward(self, x, per_layer=None):
+    def ffn_block(self, x, p, capacity, per_layer=None, index=0, table=None):
+        """The mixture-of-experts half-block (oracle/moe.py). `table` overrides the routing table computed here (used to follow the
+        device's choice where two tokens' scores are too close for two different summation orders to agree on their order)."""
+        from oracle import moe as M
+
+        b, h, w, c = x.shape
+        rows = b * h * w
+        normed = O.rmsnorm_forward(x, p["gamma"])
+        experts = np.asarray(p["w_router"]).shape[0]
+        scores = O.gemm(normed.reshape(rows, c), p["w_router"], bias=p["b_router"], act=O.LINEAR).reshape(b, h, w, experts)
+        own_table = M.expert_choice_routing(scores, capacity)
+        used = own_table if table is None else table
+        gathered = M.gather_tokens(normed, used)
+        hidden = M.moe_forward(gathered, p["w_1"], p["b_1"], O.RELU)
+        out = M.moe_forward(hidden, p["w_2"], p["b_2"], O.LINEAR)
+        scattered = M.scatter_tokens(out, used, x.shape)
+        y = O.add_tensors(np.zeros_like(x), 1.0, x, 1.0, scattered)
+        if per_layer is not None:
+            per_layer.update({"ffn_rmsnorm%d" % index: normed, "scores%d" % index: scores, "table%d" % index: own_table, "hidden%d" % index: hidden,
+                              "experts%d" % index: out, "ffn%d" % index: y})
+        return y
+
+    def forward(self, x, per_layer=None, moe_capacity=None, tables=None):
+        """moe_capacity: slots per expert; None leaves the mixture-of-experts half-blocks out. tables: optional list of routing tables
+        (one per block) to use instead of the ones computed here."""
         _, a = self.trunk.forward(x, return_trunk=True)
         if per_layer is not None:
             per_layer["trunk"] = a
         for index, p in enumerate(self.params["attention"]):
             a = self.attention_block(a, p, per_layer, index)
+            if moe_capacity is not None:
+                a = self.ffn_block(a, self.params["ffn"][index], moe_capacity, per_layer, index, None if tables is None else tables[index])
         w, b = self.params["head"]
         rows = a.shape[0] * a.shape[1] * a.shape[2]
         head = O.gemm(a.reshape(rows, a.shape[3]), w.reshape(w.shape[0], -1), bias=b, act=O.LINEAR)

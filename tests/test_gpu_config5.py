@@ -84,3 +84,79 @@ def test_config5_full_size(ctx):
     small = HybridNet(ctx, 4, BOARD, PLANES, CHANNELS, BLOCKS, HEADS, "float16", params, O.to_half)
     small.setInput(x[sample])
     assert max_abs_rel(small.forward().copyToHost(ctx), head[sample]) <= 1e-2
+
+
+# ---- the whole configuration: the mixture-of-experts halves included -------------------------------------------------------------
+
+def test_config5_with_experts_per_layer_small_batch(ctx):
+    """Batch 2 with the feed-forward halves (expert-choice routing with capacity factor 2 = 56 of 225 tokens per expert, 8 experts of
+    hidden width 1024). Every mixture-of-experts layer is checked against the CPU statement (oracle/moe.py) applied to the device's own
+    input of that layer, the routing table exactly; then the head against a CPU pass that follows the device's routing tables (two
+    summation orders may order two nearly equal scores differently; the tables themselves were just checked on identical scores)."""
+    from oracle import moe as M
+    from minml_amd.hybridnet import get_capacity
+
+    O.set_num_threads(8)
+    params = make_hybrid_parameters(SEED, PLANES, CHANNELS, BLOCKS, ATTENTION_BLOCKS, HEADS, BOARD)
+    x = O.to_half(make_input(SEED, 2, BOARD, PLANES))
+    net = HybridNet(ctx, 2, BOARD, PLANES, CHANNELS, BLOCKS, HEADS, "float16", params, O.to_half, moe=True)
+    seen = {}
+    net.observer = lambda name, tensor: seen.__setitem__(name, tensor.copyToHost(ctx))
+    net.setInput(x)
+    head = net.forward().copyToHost(ctx)
+    ps = storage_params(params)
+    ps["ffn"] = [{k: O.to_half(v) for k, v in blk.items()} for blk in params["ffn"]]
+    capacity = get_capacity(2.0, BOARD * BOARD, 8)
+    assert capacity == 56 and net.capacity == 56
+    rows = 2 * BOARD * BOARD
+    worst = {}
+    for index, p in enumerate(ps["ffn"]):
+        x_in = seen["block%d" % index]
+        worst["ffn_rmsnorm"] = max(worst.get("ffn_rmsnorm", 0.0), max_abs_rel(seen["ffn_rmsnorm%d" % index], O.rmsnorm_forward(x_in, p["gamma"])))
+        normed = seen["ffn_rmsnorm%d" % index]
+        scores = O.gemm(normed.reshape(rows, CHANNELS), p["w_router"], bias=p["b_router"], act=O.LINEAR)
+        worst["scores"] = max(worst.get("scores", 0.0), max_abs_rel(seen["scores%d" % index].reshape(rows, -1), scores))
+        table = seen["table%d" % index]
+        want_table = M.expert_choice_routing(seen["scores%d" % index], capacity)
+        assert np.array_equal(O.from_half(table)[:, 0], O.from_half(want_table)[:, 0])  # the same tokens in the same slots
+        assert np.abs(O.from_half(table)[:, 1] - O.from_half(want_table)[:, 1]).max() <= 1e-3
+        gathered = M.gather_tokens(normed, table)
+        worst["hidden"] = max(worst.get("hidden", 0.0), max_abs_rel(seen["hidden%d" % index], M.moe_forward(gathered, p["w_1"], p["b_1"], O.RELU)))
+        worst["experts"] = max(worst.get("experts", 0.0), max_abs_rel(seen["experts%d" % index], M.moe_forward(seen["hidden%d" % index], p["w_2"], p["b_2"], O.LINEAR)))
+        scattered = M.scatter_tokens(seen["experts%d" % index], table, x_in.shape)
+        want = O.add_tensors(np.zeros_like(x_in), 1.0, x_in, 1.0, scattered)
+        worst["ffn"] = max(worst.get("ffn", 0.0), max_abs_rel(seen["ffn%d" % index], want))
+    cpu = CpuHybridNet(ps, BLOCKS, HEADS)
+    want_head = cpu.forward(x, moe_capacity=capacity, tables=[seen["table%d" % i] for i in range(ATTENTION_BLOCKS)])
+    worst["head"] = max_abs_rel(head, want_head)
+    print("config 5 with experts, batch 2, max-abs relative error per layer type:", {k: "%.2e" % v for k, v in worst.items()}, flush=True)
+    assert max(worst.values()) <= 1e-2, worst
+    # every token that an expert selected moved: the feed-forward half is not a no-op
+    assert max_abs_rel(seen["ffn0"], seen["block0"]) > 1e-3
+
+
+def test_config5_with_experts_full_size(ctx):
+    """Batch 256, the complete configuration: repeatable bit for bit, finite, and the head of a sample of positions within 1e-2 of a CPU
+    pass over those positions that follows the device's routing tables."""
+    from minml_amd.hybridnet import get_capacity
+
+    O.set_num_threads(8)
+    batch = 256
+    params = make_hybrid_parameters(SEED, PLANES, CHANNELS, BLOCKS, ATTENTION_BLOCKS, HEADS, BOARD)
+    x = O.to_half(make_input(SEED, batch, BOARD, PLANES))
+    net = HybridNet(ctx, batch, BOARD, PLANES, CHANNELS, BLOCKS, HEADS, "float16", params, O.to_half, moe=True)
+    tables = {}
+    net.observer = lambda name, tensor: tables.__setitem__(name, tensor.copyToHost(ctx)) if name.startswith("table") else None
+    net.setInput(x)
+    head = net.forward().copyToHost(ctx)
+    net.observer = None
+    assert mismatches(net.forward().copyToHost(ctx), head) == 0
+    assert np.isfinite(O.from_half(head)).all()
+    sample = [0, 255]
+    ps = storage_params(params)
+    ps["ffn"] = [{k: O.to_half(v) for k, v in blk.items()} for blk in params["ffn"]]
+    cpu = CpuHybridNet(ps, BLOCKS, HEADS)
+    want = cpu.forward(x[sample], moe_capacity=get_capacity(2.0, BOARD * BOARD, 8), tables=[tables["table%d" % i][sample] for i in range(ATTENTION_BLOCKS)])
+    err = max_abs_rel(head[sample], want)
+    print("config 5 with experts, batch 256: head of positions %s vs CPU: %.2e" % (sample, err), flush=True)
+    assert err <= 1e-2
