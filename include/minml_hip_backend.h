@@ -225,6 +225,20 @@ extern "C"
 			mlQuantizationData_t output_qd, const void *ext, mlQuantizationData_t ext_qd, mlActivationType_t act);
 	/* hip_get_stream: the hipStream_t of a context, for callers that time or capture work on it. */
 	void* hip_get_stream(mlContext_t context);
+	/*
+	 * Recording a pass as a HIP graph (no counterpart in the reference, whose layers launch kernel by kernel). Between
+	 * hip_graph_begin_capture and hip_graph_end_capture the calls made on the context are recorded instead of executed;
+	 * hip_graph_launch replays them, in order, on the context's stream with one submission. For passes made of many short dependent
+	 * launches (small batches) the host's cost per launch bounds the pass, and the replay removes it. Buffers are recorded by address:
+	 * the replay reads and writes the same tensors. Record only after one ordinary pass (first-use work such as weight transforms and
+	 * workspace growth synchronises or allocates, which a recording cannot hold), and never hip_winograd_layer_errors, copies to or
+	 * from pageable host memory, or context-less (NULL) memory calls.
+	 */
+	typedef void *mlGraph_t;
+	void hip_graph_begin_capture(mlContext_t context);
+	mlGraph_t hip_graph_end_capture(mlContext_t context);
+	void hip_graph_launch(mlContext_t context, mlGraph_t graph);
+	void hip_graph_destroy(mlGraph_t graph);
 
 #ifdef __cplusplus
 }

@@ -113,6 +113,10 @@ SIGNATURES = {
     "scatter_tokens_forward": (None, [_vp, _T, _T, _f, _T]),
     "quantized_conv_forward": (None, [_vp, _S, _S, _vp, _Q, _vp, _vp, _vp, _i, _vp, _Q, _vp, _Q, _i]),
     "get_stream": (_vp, [_vp]),
+    "graph_begin_capture": (None, [_vp]),
+    "graph_end_capture": (_vp, [_vp]),
+    "graph_launch": (None, [_vp, _vp]),
+    "graph_destroy": (None, [_vp]),
 }
 
 _lib = None

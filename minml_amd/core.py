@@ -61,6 +61,37 @@ class Context:
             self.handle = None
 
 
+class Graph:
+    """A pass recorded once on a context and replayed as one HIP graph (the library's hip_graph_* calls; no counterpart in the reference).
+
+        graph = Graph.record(context, lambda: net.forward())    # after one ordinary pass
+        graph.launch()                                          # replays the recorded launches on the context's stream
+    """
+
+    def __init__(self, context, handle):
+        self.context = context
+        self.handle = handle
+
+    @staticmethod
+    def record(context, function):
+        if _TIMER is not None:
+            raise RuntimeError("a kernel timer records events around every call: remove it before recording a graph")
+        B.fn("graph_begin_capture")(context.handle)
+        try:
+            function()
+        finally:
+            handle = B.fn("graph_end_capture")(context.handle)
+        return Graph(context, handle)
+
+    def launch(self):
+        B.fn("graph_launch")(self.context.handle, self.handle)
+
+    def destroy(self):
+        if self.handle:
+            B.fn("graph_destroy")(self.handle)
+            self.handle = None
+
+
 class Event:
     """Recorded on creation (reference: include/minml/core/Event.hpp, src/backend/cuda/cuda_event.cpp)."""
 

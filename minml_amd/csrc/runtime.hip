@@ -242,6 +242,59 @@ extern "C"
 		return reinterpret_cast<void*>(stream_of(context));
 	}
 
+	/*
+	 * A sequence of calls on a context recorded once and replayed as one HIP graph: for passes that are a chain of many short dependent
+	 * launches (small batches), where the host's launch cost per kernel is what bounds the pass. Every entry point of this library only
+	 * launches kernels and copies on the context's stream, so a pass may be recorded as it is; what must not happen while recording is
+	 * anything that synchronises or allocates (first-use work such as weight transforms and workspace growth: run one pass before).
+	 */
+	struct Graph
+	{
+			int device_index = 0;
+			hipGraph_t graph = nullptr;
+			hipGraphExec_t exec = nullptr;
+	};
+	void hip_graph_begin_capture(mlContext_t context)
+	{
+		Context *ctx = get(context);
+		use_device(ctx->device_index);
+		MLHIP_CHECK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
+	}
+	mlGraph_t hip_graph_end_capture(mlContext_t context)
+	{
+		Context *ctx = get(context);
+		Graph *g = new Graph();
+		g->device_index = ctx->device_index;
+		const hipError_t status = hipStreamEndCapture(ctx->stream, &g->graph);
+		if (status != hipSuccess || g->graph == nullptr)
+		{
+			delete g;
+			check(status == hipSuccess ? hipErrorUnknown : status, "hipStreamEndCapture");
+		}
+		const hipError_t inst = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+		if (inst != hipSuccess)
+		{
+			(void) hipGraphDestroy(g->graph);
+			delete g;
+			check(inst, "hipGraphInstantiate");
+		}
+		return g;
+	}
+	void hip_graph_launch(mlContext_t context, mlGraph_t graph)
+	{
+		MLHIP_REQUIRE(graph != nullptr, "hip_graph_launch: null graph");
+		MLHIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, stream_of(context)));
+	}
+	void hip_graph_destroy(mlGraph_t graph)
+	{
+		if (graph == nullptr)
+			return;
+		Graph *g = reinterpret_cast<Graph*>(graph);
+		MLHIP_CHECK(hipGraphExecDestroy(g->exec));
+		MLHIP_CHECK(hipGraphDestroy(g->graph));
+		delete g;
+	}
+
 	mlEvent_t hip_create_event(mlContext_t context)
 	{
 		Context *ctx = get(context);

@@ -243,3 +243,31 @@ def test_network_driven_from_cpp_through_the_cabi(ctx, tmp_path, mode):
     net.setInput(x)
     want = net.forward(fused=bool(mode)).copyToHost(ctx)
     assert mismatches(got, want) == 0
+
+
+def test_recorded_pass_replays_bit_identically(ctx):
+    """A forward pass recorded as a HIP graph (hip_graph_begin_capture / end_capture / launch): every replay must equal the eager pass
+    bit for bit, also after other work and synchronisations on the same context between replays, and after the input changed in place."""
+    params = make_parameters(9, 32, 64, 3)
+    conv = O.to_half
+    net = ResNet(ctx, 8, 15, 32, 64, 3, "float16", params, conv, fused=True)
+    x1, x2 = conv(make_input(9, 8, 15, 32)), conv(make_input(10, 8, 15, 32))
+    net.setInput(x1)
+    want1 = net.forward().copyToHost(ctx)  # the ordinary pass also does the first-use work (weight transforms) outside the recording
+    graph = ml.Graph.record(ctx, lambda: net.forward())
+    for replay in range(3):
+        net.output.zeroall(ctx)
+        graph.launch()
+        assert mismatches(net.output.copyToHost(ctx), want1) == 0
+        # unrelated eager work and a synchronisation between replays
+        scratch = ml.Tensor((1024,), "float32")
+        scratch.zeroall(ctx)
+        ctx.synchronize()
+        scratch.free()
+    net.setInput(x2)
+    want2 = net.forward().copyToHost(ctx)
+    assert mismatches(want2, want1) > 0
+    net.output.zeroall(ctx)
+    graph.launch()  # same buffers, new contents
+    assert mismatches(net.output.copyToHost(ctx), want2) == 0
+    graph.destroy()
