@@ -51,12 +51,24 @@ CONFIGS = {
 }
 PEAK_INT8_TOPS = 5000.0
 
-# HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs), each counter
-# scaled by its reading for a 256 MiB copy kernel in the same run (read 324.2 MiB + written 288.1 MiB).
-# Source: profiles/hbm_traffic_cfg2_resnet20x256_fp16_b1024.md
-MEASURED_GEMM_TRAFFIC_BYTES = {
-    "cfg2_resnet20x256_fp16_b1024": 637.5e6,
-}
+def measured_gemm_traffic_bytes(config):
+    """HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each counter
+    scaled by its reading for a 256 MiB copy kernel in the same run), as recorded in profiles/hbm_traffic_<config>.md together with the
+    hash of the kernel's source file. None when there is no such record or the kernel has changed since it was measured."""
+    import hashlib
+    import re
+
+    root = os.path.dirname(os.path.abspath(__file__))
+    try:
+        text = open(os.path.join(root, "profiles", "hbm_traffic_%s.md" % config)).read()
+        m = re.search(r"kernel_gemm_stream_wide_nt traffic_bytes=(\d+) source=(\S+) sha256=([0-9a-f]{64})", text)
+        if m is None:
+            return None
+        current = hashlib.sha256(open(os.path.join(root, m.group(2)), "rb").read()).hexdigest()
+        return float(m.group(1)) if current == m.group(3) else None
+    except OSError:
+        return None
+
 
 
 def to_storage_factory(dtype):
@@ -364,7 +376,7 @@ def main():
     else:
         roofline = {"bound": "mfma", "achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s",
                     "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype]}
-    roofline.update({"traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
+    roofline.update({"traffic": measured_gemm_traffic_bytes(args.config) if net.chunk == batch else None,
                      "kernel": "%s (36 batched Winograd GEMMs, M=%d N=K=%d)" % (kernel_name, tiles, channels),
                      "algorithmic_bytes": gemm_bytes, "launches_timed": n_gemm, "avg_launch_us": t_gemm * 1e6})
     result = {
