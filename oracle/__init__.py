@@ -213,6 +213,26 @@ def quantized_scale_shift_act(acc, scales, bias, out_dtype, out_qd, ext=None, ex
     return out
 
 
+def quantized_scale_shift_act_device_form(acc, scales, bias, out_qd, ext=None, ext_qd=(1.0, 0.0), act=LINEAR):
+    """The int8 requantisation as the reference's DEVICE kernel writes it (src/backend/cuda/kernels/quantized.cu:44-47, 232-254):
+    x = acc * scale + bias (+ ext * ext_scale + ext_shift), activation, then clamp(round((x - shift) / scale)) — where the CPU layer,
+    which quantized_scale_shift_act above and the HIP library follow, evaluates clamp(round(x * (1 / scale) + (-shift / scale))).
+    PARITY UNPINNED: that kernel cannot run here, and whether its compiler contracts `acc * scale + bias` into one fused operation is
+    unknown (evaluated unfused here). Used only to count how often the two formulas disagree. int8 output, linear or ReLU."""
+    f = np.float32
+    acc = np.asarray(acc, np.int32).astype(f)
+    x = acc * np.asarray(scales, f) + np.asarray(bias, f)
+    if ext is not None:
+        x = x + (np.asarray(ext, np.int8).astype(f) * f(ext_qd[0]) + f(ext_qd[1]))
+    if act == RELU:
+        x = np.maximum(x, f(0.0))
+    elif act != LINEAR:
+        raise ValueError("linear or ReLU only")
+    q = (x - f(out_qd[1])) / f(out_qd[0])
+    q = np.sign(q) * np.floor(np.abs(q) + f(0.5))  # round(): halves away from zero
+    return np.clip(q, -128.0, 127.0).astype(np.int8)
+
+
 def quantize_weights(w, bias, in_qd):
     w = _c(w, np.float32)
     rows, cols = w.shape[0], w.size // w.shape[0]
