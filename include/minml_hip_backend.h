@@ -124,6 +124,9 @@ extern "C"
 	 * boards of 16 tiles (13x13 .. 16x16), batches that are multiples of 4 (at least 32) and linear / ReLU activation the product never
 	 * leaves the L2 cache; every other case runs the two calls through `output_matrices` [36, tiles, Cout], which must then be given.
 	 * No counterpart in the reference (src/layers/Conv2D.cpp:365-378 calls the three steps one by one).
+	 * EXPERIMENTAL, opt-in: the one-launch form assumes that the device places its 512 workgroups 64 to an XCD, all resident at once,
+	 * i.e. that nothing else runs on the GPU; it measures slower than the two calls, which remain the recommended sequence. A caller
+	 * that uses it must check hip_winograd_layer_errors after the pass.
 	 * hip_winograd_layer_errors waits for the context's stream and returns how many workgroups of such launches gave up waiting for
 	 * one another since the last call (0 unless the device was shared with other work; results are then invalid).
 	 */
