@@ -259,35 +259,147 @@ namespace
 			for (int i = 0; i < VEC; i++)
 				acc.v[i] *= beta;
 		}
-		for (int e = 0; e < experts; e++)
+		/*
+		 * Experts are taken eight at a time: first the index rows of all eight are scanned (independent loads, one ballot each per 64
+		 * slots), then their gates and rows are requested together, then the rows are added in expert order. A wavefront that looked
+		 * for one expert's slot, loaded its row and only then turned to the next expert spent its time waiting for eight chains of
+		 * dependent loads.
+		 */
+		constexpr int GROUP = 8;
+		const T *index_plane = indices_and_values + (b * 2 + 0) * experts * capacity;
+		const T *gate_plane = indices_and_values + (b * 2 + 1) * experts * capacity;
+		for (int e0 = 0; e0 < experts && capacity > 0; e0 += GROUP)
 		{
-			const T *index_row = indices_and_values + ((b * 2 + 0) * experts + e) * capacity;
+			int found[GROUP];
+#pragma unroll
+			for (int i = 0; i < GROUP; i++)
+				found[i] = -1;
 			for (int k0 = 0; k0 < capacity; k0 += 64)
 			{
-				const int k = k0 + lane;
-				const bool match = (k < capacity) && (static_cast<int>(Storage<T>::load(index_row + k)) == token);
-				const unsigned long long hits = __ballot(match);
-				if (hits != 0ull)
-				{
-					const int found = k0 + __builtin_ctzll(hits);
-					const float gate = Storage<T>::load(indices_and_values + ((b * 2 + 1) * experts + e) * capacity + found);
-					if (active)
-					{
-						Vec<T, VEC> in;
-						in.load(x + ((b * capacity + found) * experts + e) * channels + c);
+				const int k = min(k0 + lane, capacity - 1);
+				int index[GROUP];
 #pragma unroll
-						for (int i = 0; i < VEC; i++)
-						{
-							const float scaled = gate * in.v[i];
-							acc.v[i] = acc.v[i] + scaled;
-						}
-					}
-					break; /* at most one slot per expert */
+				for (int i = 0; i < GROUP; i++)
+					index[i] = static_cast<int>(Storage<T>::load(index_plane + static_cast<size_t>(min(e0 + i, experts - 1)) * capacity + k));
+#pragma unroll
+				for (int i = 0; i < GROUP; i++)
+				{
+					const unsigned long long hits = __ballot(k0 + lane < capacity && e0 + i < experts && index[i] == token);
+					if (hits != 0ull) /* at most one slot per expert holds the token */
+						found[i] = k0 + __builtin_ctzll(hits);
 				}
 			}
+			float gate[GROUP];
+			Vec<T, VEC> in[GROUP];
+#pragma unroll
+			for (int i = 0; i < GROUP; i++)
+			{
+				const int e = min(e0 + i, experts - 1), slot_k = max(found[i], 0);
+				gate[i] = Storage<T>::load(gate_plane + static_cast<size_t>(e) * capacity + slot_k);
+				in[i].zero();
+				if (active)
+					in[i].load(x + ((b * capacity + slot_k) * experts + e) * channels + c);
+			}
+#pragma unroll
+			for (int i = 0; i < GROUP; i++)
+				if (found[i] >= 0)
+				{
+#pragma unroll
+					for (int v = 0; v < VEC; v++)
+					{
+						const float scaled = gate[i] * in[i].v[v];
+						acc.v[v] = acc.v[v] + scaled;
+					}
+				}
 		}
 		if (active)
 			acc.store(y + global_token * channels + c);
+	}
+
+	/*
+	 * The same sum with the search taken out of the wavefronts' critical path. One workgroup serves a range of the tokens of ONE image:
+	 * it first inverts the image's routing table in LDS (inverse[token][expert] = the lowest slot of that expert holding the token, or
+	 * "none"), then every wavefront walks its tokens, reads a token's row of the inverse table from LDS and requests the gates and rows
+	 * of all its slots at once. Same additions in the same order as kernel_scatter_tokens, hence the same bits.
+	 */
+	constexpr int SCATTER_NONE = 0x7fffffff;
+	template<typename T, int VEC>
+	__global__ __launch_bounds__(256) void kernel_scatter_tokens_by_image(const T *x, const T *indices_and_values, T *y, float beta, int tokens, int channels,
+			int experts, int capacity, int splits)
+	{
+#pragma clang fp contract(off)
+		extern __shared__ int inverse[]; /* [tokens][experts] */
+		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+		const size_t b = blockIdx.x / splits;
+		const int part = blockIdx.x % splits;
+		const T *index_plane = indices_and_values + (b * 2 + 0) * experts * capacity;
+		const T *gate_plane = indices_and_values + (b * 2 + 1) * experts * capacity;
+		for (int i = threadIdx.x; i < tokens * experts; i += blockDim.x)
+			inverse[i] = SCATTER_NONE;
+		__syncthreads();
+		for (int i = threadIdx.x; i < experts * capacity; i += blockDim.x)
+		{
+			const int e = i / capacity, k = i - e * capacity;
+			const int token = static_cast<int>(Storage<T>::load(index_plane + i));
+			if (token >= 0 && token < tokens)
+				atomicMin(&inverse[token * experts + e], k);
+		}
+		__syncthreads();
+		const int per_part = (tokens + splits - 1) / splits;
+		const int first = part * per_part, last = min(tokens, first + per_part);
+		const int channel_blocks = (channels + 64 * VEC - 1) / (64 * VEC);
+		const int items = max(last - first, 0) * channel_blocks;
+		constexpr int GROUP = 8;
+		for (int item = wave; item < items; item += (blockDim.x >> 6))
+		{
+			const int token = first + item / channel_blocks;
+			const int c = ((item % channel_blocks) * 64 + lane) * VEC;
+			const bool active = c < channels;
+			const size_t global_token = b * tokens + token;
+			Vec<T, VEC> acc;
+			acc.zero();
+			if (beta != 0.0f && active)
+			{
+				acc.load(y + global_token * channels + c);
+#pragma unroll
+				for (int i = 0; i < VEC; i++)
+					acc.v[i] *= beta;
+			}
+			for (int e0 = 0; e0 < experts; e0 += GROUP)
+			{
+				int found[GROUP];
+				float gate[GROUP];
+				Vec<T, VEC> in[GROUP];
+#pragma unroll
+				for (int i = 0; i < GROUP; i++)
+					found[i] = (e0 + i < experts) ? __builtin_amdgcn_readfirstlane(inverse[token * experts + e0 + i]) : SCATTER_NONE;
+#pragma unroll
+				for (int i = 0; i < GROUP; i++)
+				{
+					gate[i] = 0.0f;
+					in[i].zero();
+					if (found[i] != SCATTER_NONE)
+					{
+						gate[i] = Storage<T>::load(gate_plane + static_cast<size_t>(e0 + i) * capacity + found[i]);
+						if (active)
+							in[i].load(x + ((b * capacity + found[i]) * experts + e0 + i) * channels + c);
+					}
+				}
+#pragma unroll
+				for (int i = 0; i < GROUP; i++)
+					if (found[i] != SCATTER_NONE)
+					{
+#pragma unroll
+						for (int v = 0; v < VEC; v++)
+						{
+							const float scaled = gate[i] * in[i].v[v];
+							acc.v[v] = acc.v[v] + scaled;
+						}
+					}
+			}
+			if (active)
+				acc.store(y + global_token * channels + c);
+		}
 	}
 
 	/* fallback of the expert layers for shapes the tile engine does not take: one thread per output element */
@@ -443,8 +555,18 @@ extern "C"
 			return;
 		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && indices_and_values.data != nullptr, "scatter_tokens_forward: null tensor");
 		const hipStream_t stream = stream_of(context);
+		/* the by-image form needs the inverted table of one image in LDS and a grid of (images x parts) workgroups */
+		const size_t inverse_bytes = static_cast<size_t>(tokens) * experts * sizeof(int);
+		const int splits = std::max(1, std::min(8, tokens / 16));
+		const bool by_image = experts > 0 && capacity > 0 && inverse_bytes <= 48 * 1024 && static_cast<size_t>(batch) * splits <= 0x7fffffffu;
 #define MLHIP_SCATTER(T, VEC) \
 		do { \
+			if (by_image) \
+			{ \
+				hipLaunchKernelGGL((kernel_scatter_tokens_by_image<T, VEC>), dim3(static_cast<unsigned int>(batch) * splits), dim3(256), inverse_bytes, stream, \
+						ptr<const T>(x), ptr<const T>(indices_and_values), ptr<T>(y), beta, tokens, channels, experts, capacity, splits); \
+				break; \
+			} \
 			const size_t wavefronts = total_tokens * ((channels + 64 * VEC - 1) / (64 * VEC)); \
 			MLHIP_REQUIRE((wavefronts + 3) / 4 <= 0x7fffffffu, "scatter_tokens_forward: tensor too large for one launch"); \
 			hipLaunchKernelGGL((kernel_scatter_tokens<T, VEC>), dim3(static_cast<unsigned int>((wavefronts + 3) / 4)), dim3(256), 0, stream, ptr<const T>(x), \
@@ -508,8 +630,17 @@ extern "C"
 				ep.act = act;
 				ep.vectorized = vectorized;
 				ep.bias_batch_stride = neurons;
-				launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
-						static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), ep);
+				/* the epilogue's common cases (ReLU / linear, bias present, beta = 0 or not) are fixed at compile time: with K of only a few
+				 * chunks the epilogue is most of a tile's time, and its run-time form is twice as slow */
+				if constexpr (sizeof(T) == 2)
+					specialise_epilogue(ep, [&](const auto &fixed)
+					{
+						launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
+								static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), fixed);
+					});
+				else
+					launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
+							static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), ep);
 			};
 			if (x.dtype == DTYPE_FLOAT16)
 				launch(half_t(0));

@@ -18,7 +18,7 @@ and, with `moe=True`, the feed-forward half of each transformer block as a mixtu
     g      = gather(h, table)                                 [B, K, E, C]
     u      = relu(g W_1[e]^T + b_1[e])                        MixtureOfExperts, hidden width 1024
     v      = u W_2[e]^T + b_2[e]                              MixtureOfExperts back to C
-    x      = x + scatter(v, table)                            ScatterTokens (gated sum per token), then Add
+    x      = x + scatter(v, table)                            ScatterTokens with beta = 1 (gated sum per token added to x, one rounding)
 
 and a 1x1 policy head. The reference has the mixture-of-experts kernels for its CUDA backend only (src/core/math.cpp:1328-1491
 dispatches nothing on the CPU): that half is checked against this repository's own CPU statement of those steps, not against the
@@ -86,7 +86,6 @@ class HybridNet:
             self.gathered = ml.Tensor((batch, self.capacity, self.experts, channels), self.dtype)
             self.expert_hidden = ml.Tensor((batch, self.capacity, self.experts, self.hidden), self.dtype)
             self.expert_out = ml.Tensor((batch, self.capacity, self.experts, channels), self.dtype)
-            self.scattered = ml.Tensor((batch, board, board, channels), self.dtype)
         shape = (batch, board, board, channels)
         self.head = Conv2D(context, shape, 1, 1, "linear", True, self.dtype)
         self.head.setWeights(to_storage(params["head"][0]), to_storage(params["head"][1]))
@@ -137,11 +136,9 @@ class HybridNet:
                 self._observe("hidden%d" % index, self.expert_hidden)
                 ml.moeForward(ctx, self.expert_hidden, f["w_2"], f["b_2"], 0.0, self.expert_out, "linear")
                 self._observe("experts%d" % index, self.expert_out)
-                ml.scatterTokensForward(ctx, self.expert_out, self.table, 0.0, self.scattered)
-                out = next(t for t in self.stream if t is not x)
-                ml.addTensors(ctx, 1.0, x, 1.0, self.scattered, 0.0, None, 0.0, out)
-                self._observe("ffn%d" % index, out)
-                x = out
+                # the residual addition rides on the scatter: x = 1 * x + gated sum, accumulated in fp32 and rounded once
+                ml.scatterTokensForward(ctx, self.expert_out, self.table, 1.0, x)
+                self._observe("ffn%d" % index, x)
         ml.set_timer_label("head")
         self.head.forward([x], self.output, self.workspace)
         ml.set_timer_label(None)

@@ -9,7 +9,8 @@ achieved fraction of that peak.
 Groups: winograd (transforms and batched GEMM at the residual-network shapes), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
 channels 64..384, kernels 1 / 3 / 5, bias + residual + ReLU), int8 (quantised 3x3 convolution at 256 channels and its three-call form),
 misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode), transformer
-(RMS normalisation and multi-head attention at the hybrid configuration's shape), ceilings (what the chip sustains independent of the
+(RMS normalisation and multi-head attention at the hybrid configuration's shape), moe (routing, gather, the two expert layers and
+scatter of that configuration's mixture-of-experts half-block), ceilings (what the chip sustains independent of the
 backend's kernels: read / write / copy streams over buffers that fit the L2s, the 256 MB last-level cache or neither, and a pure MFMA
 loop on constant and on random operands with the shader clock it ran at; needs libminml_ceilings.so, built by minml_amd.build).
 """
@@ -243,6 +244,40 @@ class Bench:
             for t in (x, y, gamma, qkv, table):
                 t.free()
 
+    def moe(self):
+        """The hybrid configuration's mixture-of-experts half-block: 256 images of 225 tokens, 256 channels, 8 experts of hidden width
+        1024, capacity factor 2 (56 slots per expert and image), fp16."""
+        ctx, rng = self.ctx, self.rng
+        batch, board, emb, experts, hidden, dtype, s = 256, 15, 256, 8, 1024, "float16", 2
+        tokens = board * board
+        tmp = int(2.0 * tokens / experts)
+        capacity = tmp if tmp * experts >= tokens else tmp + 1
+        tag = "cfg5 B=256 225 tokens C=256 E=8 K=%d f16" % capacity
+        x = _random(ctx, (batch, board, board, emb), dtype, rng)
+        scores = _random(ctx, (batch, board, board, experts), dtype, rng)
+        table = ml.Tensor((batch, 2, experts, capacity), dtype)
+        gathered = ml.Tensor((batch, capacity, experts, emb), dtype)
+        mid = ml.Tensor((batch, capacity, experts, hidden), dtype)
+        out = ml.Tensor((batch, capacity, experts, emb), dtype)
+        y = ml.Tensor((batch, board, board, emb), dtype)
+        w1 = _random(ctx, (experts, hidden, emb), dtype, rng, 0.02)
+        b1 = _random(ctx, (experts, hidden), dtype, rng, 0.01)
+        w2 = _random(ctx, (experts, emb, hidden), dtype, rng, 0.02)
+        b2 = _random(ctx, (experts, emb), dtype, rng, 0.01)
+        rows = batch * capacity * experts
+        self.row("moe", "expert_choice_routing_forward", tag, lambda: ml.expertChoiceRoutingForward(ctx, scores, table),
+                 s * (batch * tokens * experts + 2 * batch * experts * capacity))
+        self.row("moe", "gather_tokens_forward", tag, lambda: ml.gatherTokensForward(ctx, x, table, 0.0, gathered), s * (batch * tokens * emb + rows * emb))
+        self.row("moe", "moe_forward (256 -> 1024, relu)", tag, lambda: ml.moeForward(ctx, gathered, w1, b1, 0.0, mid, "relu"),
+                 s * (rows * emb + rows * hidden + experts * hidden * emb), 2.0 * rows * emb * hidden, dtype)
+        self.row("moe", "moe_forward (1024 -> 256, linear)", tag, lambda: ml.moeForward(ctx, mid, w2, b2, 0.0, out, "linear"),
+                 s * (rows * emb + rows * hidden + experts * hidden * emb), 2.0 * rows * emb * hidden, dtype)
+        self.row("moe", "scatter_tokens_forward", tag, lambda: ml.scatterTokensForward(ctx, out, table, 0.0, y), s * (rows * emb + batch * tokens * emb))
+        self.row("moe", "scatter_tokens_forward (beta = 1)", tag, lambda: ml.scatterTokensForward(ctx, out, table, 1.0, y),
+                 s * (rows * emb + 2 * batch * tokens * emb))
+        for t in (x, scores, table, gathered, mid, out, y, w1, b1, w2, b2):
+            t.free()
+
     def ceilings(self):
         """Plain streams and a pure MFMA loop: the ceilings the other groups' rows can be read against."""
         ctx = self.ctx
@@ -318,13 +353,13 @@ class Bench:
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "ceilings"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
-    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer", "ceilings"):
+    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"):
         if args.group in ("all", group):
             getattr(bench, group)()
     if args.json:

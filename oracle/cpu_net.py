@@ -135,8 +135,7 @@ class CpuHybridNet:
         gathered = M.gather_tokens(normed, used)
         hidden = M.moe_forward(gathered, p["w_1"], p["b_1"], O.RELU)
         out = M.moe_forward(hidden, p["w_2"], p["b_2"], O.LINEAR)
-        scattered = M.scatter_tokens(out, used, x.shape)
-        y = O.add_tensors(np.zeros_like(x), 1.0, x, 1.0, scattered)
+        y = M.scatter_tokens(out, used, x.shape, beta=1.0, y=x)  # the residual addition rides on the scatter (one rounding)
         if per_layer is not None:
             per_layer.update({"ffn_rmsnorm%d" % index: normed, "scores%d" % index: scores, "table%d" % index: own_table, "hidden%d" % index: hidden,
                               "experts%d" % index: out, "ffn%d" % index: y})

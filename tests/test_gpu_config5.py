@@ -123,8 +123,7 @@ def test_config5_with_experts_per_layer_small_batch(ctx):
         gathered = M.gather_tokens(normed, table)
         worst["hidden"] = max(worst.get("hidden", 0.0), max_abs_rel(seen["hidden%d" % index], M.moe_forward(gathered, p["w_1"], p["b_1"], O.RELU)))
         worst["experts"] = max(worst.get("experts", 0.0), max_abs_rel(seen["experts%d" % index], M.moe_forward(seen["hidden%d" % index], p["w_2"], p["b_2"], O.LINEAR)))
-        scattered = M.scatter_tokens(seen["experts%d" % index], table, x_in.shape)
-        want = O.add_tensors(np.zeros_like(x_in), 1.0, x_in, 1.0, scattered)
+        want = M.scatter_tokens(seen["experts%d" % index], table, x_in.shape, beta=1.0, y=x_in)
         worst["ffn"] = max(worst.get("ffn", 0.0), max_abs_rel(seen["ffn%d" % index], want))
     cpu = CpuHybridNet(ps, BLOCKS, HEADS)
     want_head = cpu.forward(x, moe_capacity=capacity, tables=[seen["table%d" % i] for i in range(ATTENTION_BLOCKS)])
