@@ -152,8 +152,83 @@ namespace
 	}
 }
 
+namespace
+{
+	typedef __attribute__((address_space(3))) void *lds_ptr_t;
+	typedef __attribute__((address_space(1))) const void *global_ptr_t;
+
+	/*
+	 * Operand delivery of a hypothetical one-kernel Winograd layer (batched product + output transform inside one workgroup). Such a
+	 * workgroup must hold the fp32 accumulators of ALL 36 matrix positions of its tiles: 36 x T x N x 4 bytes within ~300 KB of
+	 * registers, i.e. T x N ~ 2048 (T tiles x N output channels). It therefore fetches, per task, the rows of its T tiles (36 x T x 512
+	 * bytes at 256 channels in fp16) and the weight slice of its N columns (36 x N x 512 bytes) — the weights again for every group of T
+	 * tiles, the tile rows again for every column slice. This kernel moves exactly those operands into LDS with direct-to-LDS loads,
+	 * one matrix position per step, two steps in flight, and does nothing else (no MFMA, no LDS read, no store): its duration is a
+	 * lower bound for that design. v = [36][tiles][512 bytes], u = [36][columns][512 bytes].
+	 */
+	template<int T, int N>
+	__global__ __launch_bounds__(512) void kernel_fused_layer_operand_stream(const uint8_t *v, const uint8_t *u, int tiles, int columns, int tasks)
+	{
+		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+		constexpr int A_BLOCKS = T * 512 / 1024, B_BLOCKS = N * 512 / 1024; /* 1 KB per wavefront instruction */
+		constexpr int STEP_BYTES = (A_BLOCKS + B_BLOCKS) * 1024;
+		constexpr int LOADS = (A_BLOCKS + B_BLOCKS) / 8;
+		static_assert((A_BLOCKS + B_BLOCKS) % 8 == 0, "blocks must divide over 8 wavefronts");
+		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+		const int slices = columns / N;
+		for (int task = blockIdx.x; task < tasks; task += gridDim.x)
+		{
+			const int group = task / slices, slice = task % slices;
+			for (int p = 0; p < 36; p++)
+			{
+				uint8_t *buffer = lds + (p & 1) * STEP_BYTES;
+				const uint8_t *a = v + (static_cast<size_t>(p) * tiles + static_cast<size_t>(group) * T) * 512;
+				const uint8_t *b = u + (static_cast<size_t>(p) * columns + static_cast<size_t>(slice) * N) * 512;
+#pragma unroll
+				for (int l = 0; l < LOADS; l++)
+				{
+					const int block = wave + 8 * l;
+					const uint8_t *src = (block < A_BLOCKS) ? a + block * 1024 : b + (block - A_BLOCKS) * 1024;
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (src + lane * 16), (lds_ptr_t) (buffer + block * 1024), 16, 0, 0);
+				}
+				/* the previous step's loads have landed in every wavefront before its buffer is overwritten by the next step */
+				__builtin_amdgcn_s_waitcnt(0x0f70 | (LOADS & 15) | ((LOADS >> 4) << 14));
+				__builtin_amdgcn_s_barrier();
+			}
+		}
+		__builtin_amdgcn_s_waitcnt(0x0f70);
+	}
+}
+
 extern "C"
 {
+	/* v: 36 * tiles * 512 bytes, u: 36 * columns * 512 bytes; tile_group x column_slice is 32 x 64 or 64 x 32; returns the bytes one launch moves */
+	size_t ceil_fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups)
+	{
+		if (tiles <= 0 || columns <= 0 || tiles % tile_group != 0 || columns % column_slice != 0 || workgroups <= 0)
+			throw std::logic_error("ceilings: ceil_fused_layer_operand_stream: bad arguments");
+		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+		const int tasks = (tiles / tile_group) * (columns / column_slice);
+		const size_t lds_bytes = 2 * static_cast<size_t>(tile_group + column_slice) * 512;
+		const uint8_t *pv = reinterpret_cast<const uint8_t*>(v), *pu = reinterpret_cast<const uint8_t*>(u);
+		if (tile_group == 32 && column_slice == 64)
+		{
+			check(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_fused_layer_operand_stream<32, 64>), hipFuncAttributeMaxDynamicSharedMemorySize,
+					static_cast<int>(lds_bytes)), "hipFuncSetAttribute");
+			hipLaunchKernelGGL((kernel_fused_layer_operand_stream<32, 64>), dim3(workgroups), dim3(512), lds_bytes, s, pv, pu, tiles, columns, tasks);
+		}
+		else if (tile_group == 64 && column_slice == 32)
+		{
+			check(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_fused_layer_operand_stream<64, 32>), hipFuncAttributeMaxDynamicSharedMemorySize,
+					static_cast<int>(lds_bytes)), "hipFuncSetAttribute");
+			hipLaunchKernelGGL((kernel_fused_layer_operand_stream<64, 32>), dim3(workgroups), dim3(512), lds_bytes, s, pv, pu, tiles, columns, tasks);
+		}
+		else
+			throw std::logic_error("ceilings: ceil_fused_layer_operand_stream: 32 x 64 or 64 x 32 only");
+		check(hipGetLastError(), "launch of kernel_fused_layer_operand_stream");
+		return static_cast<size_t>(tasks) * 36 * static_cast<size_t>(tile_group + column_slice) * 512;
+	}
+
 	/* mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16; nt != 0 uses non-temporal accesses */
 	void ceil_stream(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
 	{

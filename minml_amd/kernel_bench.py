@@ -290,6 +290,8 @@ class Bench:
         lib.ceil_stream.restype = None
         lib.ceil_mfma.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
         lib.ceil_mfma.restype = None
+        lib.ceil_fused_layer_operand_stream.argtypes = [vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        lib.ceil_fused_layer_operand_stream.restype = ctypes.c_size_t
         stream = ctx.stream()
         mib = 1 << 20
 
@@ -332,6 +334,18 @@ class Bench:
             report("copy chain over 3 buffers", "3 x %d MiB" % size_mib, self.time(step), 2 * nbytes)
             for t in bufs:
                 t.free()
+        # operand delivery of a one-kernel Winograd layer at the 20 x 256 network's shape (16384 tiles, 256 -> 256 channels, fp16)
+        tiles, columns = 16384, 256
+        v = ml.Tensor((36 * tiles * 512,), "uint8")
+        u = ml.Tensor((36 * columns * 512,), "uint8")
+        v.zeroall(ctx)
+        u.zeroall(ctx)
+        for group, width in ((32, 64), (64, 32)):
+            moved = []
+            t = self.time(lambda: moved.append(lib.ceil_fused_layer_operand_stream(stream, v.ptr, u.ptr, tiles, columns, group, width, 256)))
+            report("one-kernel Winograd layer: operands", "%d tiles x %d columns x 36 per task" % (group, width), t, moved[-1])
+        v.free()
+        u.free()
         out8 = ml.Tensor((4096,), "uint8")
         iters, wgs = 20000, 256
         for int8, name, peak, ops_per_mfma in ((0, "v_mfma_f32_32x32x16_f16", PEAK["float16"], 2.0 * 32 * 32 * 16),
