@@ -243,6 +243,20 @@ extern "C"
 	void hip_graph_launch(mlContext_t context, mlGraph_t graph);
 	void hip_graph_destroy(mlGraph_t graph);
 
+	/*
+	 * Error capture for hosts that cannot catch C++ exceptions (no counterpart in the reference, whose only callers are C++). Every entry
+	 * point above reports errors by throwing std::logic_error / std::runtime_error, as the reference's backends do. After
+	 * hip_set_error_capture(1) an entry point that fails records the exception instead, returns normally (zero / null where it returns
+	 * a value) and has done none of its work; hip_take_last_error copies the message of the first failure since its last call into
+	 * `buffer` (at most size - 1 characters), clears it and returns 0 (no failure), 1 (std::logic_error: a bad argument), 2
+	 * (std::runtime_error: the device or the runtime refused) or 3 (anything else). hip_error_flag_address returns the address of the
+	 * int that holds that code (non-zero while a failure waits to be taken), for hosts that want to test it without a call.
+	 * Process-wide; off by default.
+	 */
+	void hip_set_error_capture(int enabled);
+	int hip_take_last_error(char *buffer, int size);
+	const int* hip_error_flag_address(void);
+
 #ifdef __cplusplus
 }
 #endif

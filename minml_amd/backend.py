@@ -117,6 +117,9 @@ SIGNATURES = {
     "graph_end_capture": (_vp, [_vp]),
     "graph_launch": (None, [_vp, _vp]),
     "graph_destroy": (None, [_vp]),
+    "set_error_capture": (None, [_i]),
+    "take_last_error": (_i, [ctypes.c_char_p, _i]),
+    "error_flag_address": (_vp, []),
 }
 
 _lib = None
@@ -134,9 +137,39 @@ def load():
             fn = getattr(lib, "hip_" + name)
             fn.restype = restype
             fn.argtypes = argtypes
+        # exceptions cannot unwind through ctypes: the library records failures instead and fn()'s wrappers raise them
+        lib.hip_set_error_capture(1)
+        global _error_flag
+        _error_flag = ctypes.c_int.from_address(lib.hip_error_flag_address())
         _lib = lib
     return _lib
 
 
+_error_flag = None
+_error_buffer = ctypes.create_string_buffer(2048)
+_checked = {}
+
+
+def check_error():
+    """Raises what a library call recorded: ValueError for a std::logic_error (a bad argument), RuntimeError otherwise."""
+    kind = _lib.hip_take_last_error(_error_buffer, 2048)
+    if kind != 0:
+        message = _error_buffer.value.decode("utf-8", "replace")
+        raise (ValueError if kind == 1 else RuntimeError)(message)
+
+
 def fn(name):
-    return getattr(load(), "hip_" + name)
+    """The entry point hip_<name>, wrapped so that a failure inside the library surfaces as a Python exception."""
+    wrapped = _checked.get(name)
+    if wrapped is None:
+        raw = getattr(load(), "hip_" + name)
+        flag = _error_flag
+
+        def wrapped(*args):
+            result = raw(*args)
+            if flag.value != 0:
+                check_error()
+            return result
+
+        _checked[name] = wrapped
+    return wrapped

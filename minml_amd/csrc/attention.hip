@@ -590,6 +590,7 @@ extern "C"
 	using namespace mlhip;
 
 	void hip_rmsnorm_forward(mlContext_t context, mlShape_t shape, mlDataType_t dtype, const void *input, void *output, const void *weights)
+	try
 	{
 		if (volume(shape) == 0)
 			return;
@@ -610,10 +611,15 @@ extern "C"
 				fail_logic("HIP backend: rmsnorm_forward: unsupported data type");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	/* elements of the caller's workspace: inference needs none here (the scores never leave the chip); the training count is the
 	 * reference's (src/backend/cuda/kernels/attention.cu, src/backend/cpu/attention.cpp:303-313) for callers that size buffers by it */
 	int hip_multi_head_attention_get_workspace_size(mlShape_t input_shape, mlShape_t weights_shape, int num_heads, bool training)
+	try
 	{
 		if (!training)
 			return 0;
@@ -621,9 +627,14 @@ extern "C"
 		const int tokens = input_shape.dim[1] * input_shape.dim[2];
 		return 2 * input_shape.dim[0] * num_heads * tokens * tokens;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<int>();
+	}
 
 	void hip_multi_head_attention_forward(mlContext_t context, mlShape_t input_shape, mlShape_t weights_shape, mlShape_t bias_shape, mlDataType_t dtype,
 			const void *input, void *output, const void *weights, const void *bias, void *workspace, void *backward_data, int num_heads, bool symmetric)
+	try
 	{
 		MLHIP_REQUIRE(input_shape.rank == 4, "multi_head_attention_forward: input must be [B, H, W, C]");
 		MLHIP_REQUIRE(num_heads > 0, "multi_head_attention_forward: number of heads must be positive");
@@ -669,6 +680,10 @@ extern "C"
 			default:
 				fail_logic("HIP backend: multi_head_attention_forward: unsupported data type");
 		}
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 
 	MLHIP_ALSO_AS_CUDA(rmsnorm_forward)

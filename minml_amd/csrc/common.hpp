@@ -14,6 +14,7 @@
 #include <cstddef>
 #include <stdexcept>
 #include <string>
+#include <type_traits>
 
 namespace mlhip
 {
@@ -30,6 +31,22 @@ namespace mlhip
 			int device_index = 0;
 			hipEvent_t event = nullptr;
 	};
+
+	/*
+	 * Errors leave every entry point as C++ exceptions, as in the reference. A host that cannot catch them (ctypes and other C FFIs: the
+	 * exception would end the process) switches capture on with hip_set_error_capture(1): the entry point then records the exception,
+	 * returns normally (a zero / null value where it returns one), and the host asks hip_take_last_error afterwards. Every entry point
+	 * is a function-try-block whose handler calls entry_failed; with capture off the handler rethrows and nothing changes.
+	 */
+	bool capture_current_exception(); /* runtime.hip; call from a catch handler only */
+	template<typename R>
+	inline R entry_failed()
+	{
+		if (!capture_current_exception())
+			throw;
+		if constexpr (!std::is_void<R>::value)
+			return R();
+	}
 
 	[[noreturn]] inline void fail_runtime(const std::string &msg)
 	{

@@ -232,6 +232,7 @@ extern "C"
 
 	void hip_convolution_implicit_gemm_forward(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, mlShape_t weights_shape,
 			const void *input, const void *weights, void *output, const void *bias, const void *add, mlActivationType_t act)
+	try
 	{
 		MLHIP_REQUIRE(input_shape.rank == 4 && weights_shape.rank == 4, "convolution: input must be [B,H,W,Cin] and weights [Cout,k,k,Cin]");
 		MLHIP_REQUIRE(input_shape.dim[3] == weights_shape.dim[3], "convolution: input and weights disagree on the number of input filters");
@@ -244,9 +245,14 @@ extern "C"
 		else
 			conv_forward<float>(stream_of(context), dtype, input_shape, weights_shape, input, weights, output, bias, add, act);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	void hip_im2row(mlContext_t context, mlDataType_t dtype, mlShape_t input_shape, void *output, const void *input, int kernel_size, bool invert,
 			const void *padding)
+	try
 	{
 		MLHIP_REQUIRE(input_shape.rank == 4, "im2row: input must be [B,H,W,C]");
 		MLHIP_REQUIRE(kernel_size >= 1, "im2row: kernel size must be positive");
@@ -301,6 +307,10 @@ extern "C"
 					break;
 				}
 			}
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

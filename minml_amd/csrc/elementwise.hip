@@ -229,6 +229,7 @@ extern "C"
 	using namespace mlhip;
 
 	void hip_add_bias_act(mlContext_t context, float alpha, const mlTensor_t x, const mlTensor_t b, float beta, mlTensor_t y, mlActivationType_t act)
+	try
 	{
 		if (volume(x) == 0)
 			return;
@@ -249,7 +250,12 @@ extern "C"
 				fail_logic("HIP backend: add_bias_act: unsupported data type");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_activation_forward(mlContext_t context, float alpha, const mlTensor_t x, float beta, mlTensor_t y, mlActivationType_t act)
+	try
 	{
 		if (volume(x) == 0)
 			return;
@@ -273,8 +279,13 @@ extern "C"
 		/* one row of all elements: the widest vector form that divides the length applies */
 		hip_add_bias_act(context, alpha, flat, no_bias, beta, flat_y, act);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_add_tensors(mlContext_t context, float alpha1, const mlTensor_t x1, float alpha2, const mlTensor_t x2, float alpha3, const mlTensor_t x3,
 			float beta, mlTensor_t y)
+	try
 	{
 		if (volume(y) == 0 || y.data == nullptr)
 			return;
@@ -291,6 +302,10 @@ extern "C"
 				fail_logic("HIP backend: add_tensors: unsupported data type");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_scale_tensor(mlContext_t context, float alpha, mlTensor_t x)
 	{ /* x *= alpha (reference: src/backend/cuda/kernels/tensor_op.cu:318-321) */
 		mlTensor_t none;
@@ -300,6 +315,7 @@ extern "C"
 		hip_add_tensors(context, 0.0f, none, 0.0f, none, 0.0f, none, alpha, x);
 	}
 	void hip_convert_type(mlContext_t context, void *dst, mlDataType_t dst_dtype, const void *src, mlDataType_t src_dtype, int elements)
+	try
 	{
 		if (elements <= 0)
 			return;
@@ -319,7 +335,12 @@ extern "C"
 			fail_logic("unsupported conversion");
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_unpack_input(mlContext_t context, mlShape_t shape, mlDataType_t dst_dtype, void *dst, const void *src)
+	try
 	{
 		if (volume(shape) == 0)
 			return;
@@ -352,6 +373,10 @@ extern "C"
 				fail_logic("HIP backend: unpack_input: unsupported destination type");
 		}
 		MLHIP_CHECK(hipGetLastError());
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

@@ -13,6 +13,8 @@
  * a plain one-thread-per-output kernel that is correct for every case and makes no performance claim.
  */
 #include "common.hpp"
+
+#include <algorithm>
 #include "gemm_core.hpp"
 #include "epilogues.hpp"
 #include "gemm_launch.hpp"
@@ -107,7 +109,22 @@ namespace mlhip
 			return;
 		MLHIP_REQUIRE(g.A != nullptr && g.B != nullptr && g.D != nullptr, "gemm: null matrix");
 		MLHIP_REQUIRE(g.beta == 0.0f || g.C != nullptr, "gemm: beta != 0 needs a C matrix");
-		MLHIP_REQUIRE(g.batch <= 65535, "gemm: at most 65535 matrices in a batch");
+		if (g.batch > 65535)
+		{ /* the matrix index rides in the grid's second dimension: longer batches go slice by slice */
+			const int esize_in = size_of(g.dtype), esize_out = (g.dtype == DTYPE_INT8) ? 4 : esize_in;
+			for (int first = 0; first < g.batch; first += 65535)
+			{
+				GemmArgs part = g;
+				part.batch = std::min(65535, g.batch - first);
+				part.A = reinterpret_cast<const uint8_t*>(g.A) + static_cast<size_t>(first) * g.stride_a * esize_in;
+				part.B = reinterpret_cast<const uint8_t*>(g.B) + static_cast<size_t>(first) * g.stride_b * esize_in;
+				part.D = reinterpret_cast<uint8_t*>(g.D) + static_cast<size_t>(first) * g.stride_c * esize_out;
+				if (g.C != nullptr)
+					part.C = reinterpret_cast<const uint8_t*>(g.C) + static_cast<size_t>(first) * g.stride_c * esize_out;
+				launch_gemm(stream, part);
+			}
+			return;
+		}
 
 		const int esize = size_of(g.dtype);
 		const bool nt = !g.transpose_a && g.transpose_b;
@@ -312,6 +329,7 @@ extern "C"
 
 	void hip_gemm(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
 			const void *B, char opA, char opB, float alpha, float beta)
+	try
 	{
 		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_C, false);
 		g.A = A;
@@ -322,8 +340,13 @@ extern "C"
 		g.beta = beta;
 		run_gemm(context, g);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_gemm_batched(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
 			const void *B, char opA, char opB, float alpha, float beta)
+	try
 	{
 		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_C, true);
 		g.A = A;
@@ -334,7 +357,12 @@ extern "C"
 		g.beta = beta;
 		run_gemm(context, g);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
+	try
 	{
 		mlDataType_t dtype = C.dtype;
 		if (C.dtype == DTYPE_INT32)
@@ -347,14 +375,24 @@ extern "C"
 			MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm: A, B and C must have one data type");
 		hip_gemm(context, dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_gemm_batched_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
+	try
 	{
 		MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm_batched: A, B and C must have one data type");
 		MLHIP_REQUIRE(C.dtype == DTYPE_FLOAT16 || C.dtype == DTYPE_FLOAT32, "gemm_batched: unsupported data type");
 		hip_gemm_batched(context, C.dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_gemm_ex(mlContext_t context, mlDataType_t dtype, mlShape_t shape_D, void *D, float alpha, char opA, mlShape_t shape_A, const void *A,
 			char opB, mlShape_t shape_B, const void *B, float beta, mlShape_t shape_C, const void *C, const void *bias, mlActivationType_t act)
+	try
 	{
 		MLHIP_REQUIRE(dtype == DTYPE_FLOAT16 || dtype == DTYPE_FLOAT32, "gemm_ex: unsupported data type");
 		GemmArgs g = make_gemm_args(dtype, opA, opB, shape_A, shape_B, shape_D, false);
@@ -369,6 +407,10 @@ extern "C"
 		g.bias = bias;
 		g.act = act;
 		run_gemm(context, g);
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

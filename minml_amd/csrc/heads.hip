@@ -18,6 +18,7 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <algorithm>
 #include <cmath>
 
 namespace
@@ -393,6 +394,7 @@ extern "C"
 	using namespace mlhip;
 
 	void hip_softmax_forward(mlContext_t context, mlDataType_t dtype, mlShape_t shape, void *output, const void *input)
+	try
 	{
 		if (volume(shape) == 0)
 			return;
@@ -411,7 +413,12 @@ extern "C"
 				fail_logic("HIP backend: softmax_forward: unsupported data type");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_global_average_pooling_forward(mlContext_t context, float alpha, const mlTensor_t x, float beta, mlTensor_t y)
+	try
 	{
 		MLHIP_REQUIRE(x.rank == 4 && y.rank == 2, "global_average_pooling_forward: x must be [B, H, W, C] and y [B, C]");
 		MLHIP_REQUIRE(x.dim[0] == y.dim[0] && x.dim[3] == y.dim[1], "global_average_pooling_forward: x and y disagree in batch or channels");
@@ -420,22 +427,28 @@ extern "C"
 			return;
 		MLHIP_REQUIRE(x.dim[1] > 0 && x.dim[2] > 0, "global_average_pooling_forward: empty spatial extent");
 		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr, "global_average_pooling_forward: null tensor");
-		MLHIP_REQUIRE(x.dim[0] <= 65535, "global_average_pooling_forward: more than 65535 images in one call");
-		mlTensor_t out = y;
-		switch (x.dtype)
+		MLHIP_REQUIRE(x.dtype == DTYPE_FLOAT16 || x.dtype == DTYPE_FLOAT32, "global_average_pooling_forward: unsupported data type");
+		/* the image index rides in the grid's second dimension: longer batches go slice by slice */
+		const size_t esize = size_of(x.dtype), image = static_cast<size_t>(x.dim[1]) * x.dim[2] * x.dim[3] * esize, row = static_cast<size_t>(x.dim[3]) * esize;
+		for (int first = 0; first < x.dim[0]; first += 65535)
 		{
-			case DTYPE_FLOAT16:
-				launch_pooling<half_t>(stream_of(context), alpha, x, beta, out);
-				break;
-			case DTYPE_FLOAT32:
-				launch_pooling<float>(stream_of(context), alpha, x, beta, out);
-				break;
-			default:
-				fail_logic("HIP backend: global_average_pooling_forward: unsupported data type");
+			mlTensor_t in = x, out = y;
+			in.dim[0] = out.dim[0] = std::min(65535, x.dim[0] - first);
+			in.data = reinterpret_cast<uint8_t*>(x.data) + first * image;
+			out.data = reinterpret_cast<uint8_t*>(y.data) + first * row;
+			if (x.dtype == DTYPE_FLOAT16)
+				launch_pooling<half_t>(stream_of(context), alpha, in, beta, out);
+			else
+				launch_pooling<float>(stream_of(context), alpha, in, beta, out);
 		}
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 	void hip_batchnorm_inference(mlContext_t context, float alpha, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, const mlTensor_t avg_var,
 			float beta, mlTensor_t y, mlActivationType_t act)
+	try
 	{
 		if (volume(x) == 0)
 			return;
@@ -461,8 +474,13 @@ extern "C"
 				fail_logic("HIP backend: batchnorm_inference: unsupported data type");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_fold_batchnorm(mlContext_t context, mlTensor_t layer_weights, mlTensor_t layer_bias, const mlTensor_t bn_weights, const mlTensor_t bn_bias,
 			const mlTensor_t bn_avg_var)
+	try
 	{
 		if (volume(layer_weights) == 0)
 			return;
@@ -499,6 +517,10 @@ extern "C"
 				fail_logic("HIP backend: fold_batchnorm: unsupported data type");
 		}
 		MLHIP_CHECK(hipGetLastError());
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

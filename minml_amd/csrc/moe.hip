@@ -459,6 +459,7 @@ extern "C"
 	using namespace mlhip;
 
 	void hip_expert_choice_routing_forward(mlContext_t context, const mlTensor_t x, mlTensor_t indices_and_values)
+	try
 	{
 		require_routing_tensors(x, indices_and_values, "expert_choice_routing_forward");
 		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
@@ -474,7 +475,12 @@ extern "C"
 					tokens, experts, capacity);
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_token_choice_routing_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t bias, mlTensor_t indices_and_values)
+	try
 	{
 		require_routing_tensors(x, indices_and_values, "token_choice_routing_forward");
 		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
@@ -491,7 +497,12 @@ extern "C"
 					ptr<float>(indices_and_values), tokens, experts, capacity);
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_hash_routing(mlContext_t context, const mlTensor_t x, mlTensor_t indices_and_values)
+	try
 	{
 		require_routing_tensors(x, indices_and_values, "hash_routing");
 		const int batch = x.dim[0], tokens = x.dim[1] * x.dim[2], experts = x.dim[3], capacity = indices_and_values.dim[3];
@@ -507,8 +518,13 @@ extern "C"
 					experts, capacity);
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	void hip_gather_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta, mlTensor_t y)
+	try
 	{
 		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && indices_and_values.rank == 4 && indices_and_values.dim[1] == 2,
 				"gather_tokens_forward: x [B, H, W, C], routing table [B, 2, E, K], y [B, K, E, C]");
@@ -541,7 +557,12 @@ extern "C"
 #undef MLHIP_GATHER
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_scatter_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta, mlTensor_t y)
+	try
 	{
 		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && indices_and_values.rank == 4 && indices_and_values.dim[1] == 2,
 				"scatter_tokens_forward: x [B, K, E, C], routing table [B, 2, E, K], y [B, H, W, C]");
@@ -589,8 +610,13 @@ extern "C"
 #undef MLHIP_SCATTER
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	void hip_moe_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, float beta, mlTensor_t y, mlActivationType_t act)
+	try
 	{
 		MLHIP_REQUIRE(x.rank == 4 && y.rank == 4 && w.rank == 3, "moe_forward: x [B, K, E, C], weights [E, N, C], y [B, K, E, N]");
 		const int batch = x.dim[0], capacity = x.dim[1], experts = x.dim[2], channels = x.dim[3], neurons = w.dim[1];
@@ -658,6 +684,10 @@ extern "C"
 						ptr<const float>(b), ptr<float>(y), beta, outputs, experts, neurons, channels, static_cast<int>(act));
 		}
 		MLHIP_CHECK(hipGetLastError());
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

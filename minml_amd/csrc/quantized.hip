@@ -234,6 +234,7 @@ extern "C"
 
 	void hip_quantized_scale_shift_act(mlContext_t context, mlDataType_t dtype, mlShape_t shape, void *output, mlQuantizationData_t output_qd,
 			const void *input, const void *scales, const void *bias, mlActivationType_t act, const void *ext, mlQuantizationData_t ext_qd)
+	try
 	{
 		MLHIP_REQUIRE(shape.rank >= 1, "quantized_scale_shift_act: empty shape");
 		if (volume(shape) == 0)
@@ -254,10 +255,15 @@ extern "C"
 				fail_logic("HIP backend: quantized_scale_shift_act: output must be INT8, FLOAT16 or FLOAT32");
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	void hip_quantized_conv_forward(mlContext_t context, mlShape_t input_shape, mlShape_t weights_shape, const void *input,
 			mlQuantizationData_t input_qd, const void *weights, const void *scales, const void *bias, mlDataType_t output_dtype, void *output,
 			mlQuantizationData_t output_qd, const void *ext, mlQuantizationData_t ext_qd, mlActivationType_t act)
+	try
 	{
 		MLHIP_REQUIRE(input_shape.rank == 4 && weights_shape.rank == 4, "quantized convolution: input must be [B,H,W,Cin] and weights [Cout,k,k,Cin]");
 		MLHIP_REQUIRE(input_shape.dim[3] == weights_shape.dim[3], "quantized convolution: input and weights disagree on the number of input filters");
@@ -276,6 +282,10 @@ extern "C"
 			default:
 				fail_logic("HIP backend: quantized convolution: output must be INT8 or FLOAT32");
 		}
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

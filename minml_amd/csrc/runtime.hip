@@ -4,6 +4,8 @@
  */
 #include "common.hpp"
 
+#include <algorithm>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <map>
@@ -153,21 +155,97 @@ namespace mlhip
 	}
 }
 
+namespace mlhip
+{
+	namespace
+	{
+		std::atomic<int> error_capture { 0 };
+		std::mutex error_mutex;
+		int error_kind = 0; /* 0 none, 1 std::logic_error, 2 std::runtime_error or another std::exception, 3 anything else */
+		std::string error_message;
+	}
+	bool capture_current_exception()
+	{
+		if (error_capture.load() == 0)
+			return false;
+		int kind = 3;
+		std::string message = "unknown exception";
+		try
+		{
+			throw;
+		}
+		catch (const std::logic_error &e)
+		{
+			kind = 1;
+			message = e.what();
+		}
+		catch (const std::exception &e)
+		{
+			kind = 2;
+			message = e.what();
+		}
+		catch (...)
+		{
+		}
+		std::lock_guard<std::mutex> lock(error_mutex);
+		if (error_kind == 0)
+		{ /* the first failure since the last hip_take_last_error is the one reported */
+			error_kind = kind;
+			error_message = message;
+		}
+		return true;
+	}
+}
+
 extern "C"
 {
+	void hip_set_error_capture(int enabled)
+	{
+		mlhip::error_capture.store(enabled != 0 ? 1 : 0);
+	}
+	const int* hip_error_flag_address(void)
+	{
+		return &mlhip::error_kind;
+	}
+	int hip_take_last_error(char *buffer, int size)
+	{
+		std::lock_guard<std::mutex> lock(mlhip::error_mutex);
+		const int kind = mlhip::error_kind;
+		if (buffer != nullptr && size > 0)
+		{
+			const size_t n = std::min(static_cast<size_t>(size - 1), mlhip::error_message.size());
+			std::memcpy(buffer, mlhip::error_message.data(), n);
+			buffer[n] = 0;
+		}
+		mlhip::error_kind = 0;
+		mlhip::error_message.clear();
+		return kind;
+	}
+
 	using namespace mlhip;
 
 	int hip_get_number_of_devices(void)
+	try
 	{
 		return static_cast<int>(device_properties().size());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<int>();
+	}
 	int hip_get_memory(int index)
+	try
 	{
 		if (index < 0 || index >= hip_get_number_of_devices())
 			return 0;
 		return static_cast<int>(device_properties()[index].totalGlobalMem >> 20);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<int>();
+	}
 	bool hip_supports_type(int index, mlDataType_t dtype)
+	try
 	{
 		if (index < 0 || index >= hip_get_number_of_devices())
 			return false;
@@ -182,25 +260,45 @@ extern "C"
 				return false;
 		}
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<bool>();
+	}
 	const char* hip_get_device_info(int index)
+	try
 	{
 		if (index < 0 || index >= hip_get_number_of_devices())
 			return nullptr;
 		return device_infos()[index].c_str();
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<const char*>();
+	}
 	const char* hip_get_device_features(int index)
+	try
 	{
 		if (index < 0 || index >= hip_get_number_of_devices())
 			return nullptr;
 		return device_features()[index].c_str();
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<const char*>();
+	}
 	void hip_enable_tf32(mlContext_t context, bool b)
+	try
 	{
 		(void) context;
 		(void) b;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	mlContext_t hip_create_context(int device_index)
+	try
 	{
 		if (device_index < 0 || device_index >= hip_get_number_of_devices())
 			fail_logic("HIP backend: hip_create_context: no such device");
@@ -211,11 +309,21 @@ extern "C"
 		MLHIP_CHECK(hipStreamCreate(&ctx->stream));
 		return ctx;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<mlContext_t>();
+	}
 	void hip_synchronize_with_context(mlContext_t context)
+	try
 	{
 		MLHIP_CHECK(hipStreamSynchronize(stream_of(context)));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	bool hip_is_context_ready(mlContext_t context)
+	try
 	{
 		const hipError_t status = hipStreamQuery(stream_of(context));
 		if (status == hipSuccess)
@@ -225,7 +333,12 @@ extern "C"
 		check(status, "hipStreamQuery");
 		return false;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<bool>();
+	}
 	void hip_destroy_context(mlContext_t context)
+	try
 	{
 		if (context == nullptr)
 			return;
@@ -237,9 +350,18 @@ extern "C"
 		MLHIP_CHECK(hipStreamDestroy(ctx->stream));
 		delete ctx;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void* hip_get_stream(mlContext_t context)
+	try
 	{
 		return reinterpret_cast<void*>(stream_of(context));
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void*>();
 	}
 
 	/*
@@ -255,12 +377,18 @@ extern "C"
 			hipGraphExec_t exec = nullptr;
 	};
 	void hip_graph_begin_capture(mlContext_t context)
+	try
 	{
 		Context *ctx = get(context);
 		use_device(ctx->device_index);
 		MLHIP_CHECK(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeThreadLocal));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	mlGraph_t hip_graph_end_capture(mlContext_t context)
+	try
 	{
 		Context *ctx = get(context);
 		Graph *g = new Graph();
@@ -280,12 +408,22 @@ extern "C"
 		}
 		return g;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<mlGraph_t>();
+	}
 	void hip_graph_launch(mlContext_t context, mlGraph_t graph)
+	try
 	{
 		MLHIP_REQUIRE(graph != nullptr, "hip_graph_launch: null graph");
 		MLHIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, stream_of(context)));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_graph_destroy(mlGraph_t graph)
+	try
 	{
 		if (graph == nullptr)
 			return;
@@ -294,8 +432,13 @@ extern "C"
 		MLHIP_CHECK(hipGraphDestroy(g->graph));
 		delete g;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	mlEvent_t hip_create_event(mlContext_t context)
+	try
 	{
 		Context *ctx = get(context);
 		use_device(ctx->device_index);
@@ -305,19 +448,34 @@ extern "C"
 		MLHIP_CHECK(hipEventRecord(ev->event, ctx->stream));
 		return ev;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<mlEvent_t>();
+	}
 	double hip_get_time_between_events(mlEvent_t start, mlEvent_t end)
+	try
 	{
 		MLHIP_REQUIRE(start != nullptr && end != nullptr, "null event");
 		float ms = 0.0f;
 		MLHIP_CHECK(hipEventElapsedTime(&ms, reinterpret_cast<Event*>(start)->event, reinterpret_cast<Event*>(end)->event));
 		return static_cast<double>(ms) * 1.0e-3;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<double>();
+	}
 	void hip_wait_for_event(mlEvent_t event)
+	try
 	{
 		MLHIP_REQUIRE(event != nullptr, "null event");
 		MLHIP_CHECK(hipEventSynchronize(reinterpret_cast<Event*>(event)->event));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	bool hip_is_event_ready(mlEvent_t event)
+	try
 	{
 		MLHIP_REQUIRE(event != nullptr, "null event");
 		const hipError_t status = hipEventQuery(reinterpret_cast<Event*>(event)->event);
@@ -328,7 +486,12 @@ extern "C"
 		check(status, "hipEventQuery");
 		return false;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<bool>();
+	}
 	void hip_destroy_event(mlEvent_t event)
+	try
 	{
 		if (event == nullptr)
 			return;
@@ -336,8 +499,13 @@ extern "C"
 		MLHIP_CHECK(hipEventDestroy(ev->event));
 		delete ev;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 
 	void* hip_malloc(int device_index, size_t count)
+	try
 	{
 		if (count == 0)
 			return nullptr;
@@ -346,32 +514,62 @@ extern "C"
 		MLHIP_CHECK(hipMalloc(&result, count));
 		return result;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void*>();
+	}
 	void hip_page_lock(void *ptr, size_t count)
+	try
 	{
 		(void) ptr;
 		(void) count;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_page_unlock(void *ptr)
+	try
 	{
 		(void) ptr;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_free(void *ptr)
+	try
 	{
 		if (ptr != nullptr)
 			MLHIP_CHECK(hipFree(ptr));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void* hip_create_view(void *src, size_t offset, size_t count)
+	try
 	{
 		(void) count;
 		if (src == nullptr)
 			return nullptr;
 		return reinterpret_cast<uint8_t*>(src) + offset;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void*>();
+	}
 	void hip_destroy_view(void *ptr)
+	try
 	{
 		(void) ptr;
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_memset(mlContext_t context, void *dst, size_t dst_offset, size_t dst_count, const void *src, size_t src_count)
+	try
 	{
 		MLHIP_REQUIRE(dst != nullptr, "hip_memset: null destination");
 		if (dst_count == 0)
@@ -411,7 +609,12 @@ extern "C"
 		if (context == nullptr)
 			MLHIP_CHECK(hipDeviceSynchronize());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_memcpy_within_device(mlContext_t context, void *dst, size_t dst_offset, const void *src, size_t src_offset, size_t count)
+	try
 	{
 		if (count == 0)
 			return;
@@ -423,7 +626,12 @@ extern "C"
 		else
 			MLHIP_CHECK(hipMemcpyAsync(d, s, count, hipMemcpyDeviceToDevice, stream_of(context)));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_memcpy_from_host(mlContext_t context, void *dst, size_t dst_offset, const void *src, size_t count)
+	try
 	{
 		if (count == 0)
 			return;
@@ -434,7 +642,12 @@ extern "C"
 		else
 			MLHIP_CHECK(hipMemcpyAsync(d, src, count, hipMemcpyHostToDevice, stream_of(context)));
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_memcpy_to_host(mlContext_t context, void *dst, const void *src, size_t src_offset, size_t count)
+	try
 	{
 		if (count == 0)
 			return;
@@ -444,6 +657,10 @@ extern "C"
 			MLHIP_CHECK(hipMemcpy(dst, s, count, hipMemcpyDeviceToHost));
 		else
 			MLHIP_CHECK(hipMemcpyAsync(dst, s, count, hipMemcpyDeviceToHost, stream_of(context)));
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 } /* extern "C" */
 

@@ -1184,6 +1184,7 @@ extern "C"
 	using namespace mlhip;
 
 	void hip_winograd_weight_transform(mlContext_t context, int tile_size, const mlTensor_t w, mlTensor_t matrices, bool invert)
+	try
 	{
 		MLHIP_REQUIRE(w.rank == 4 && w.dim[1] == w.dim[2], "Winograd weights must be [Cout, k, k, Cin] with a square kernel");
 		require_supported(tile_size, matrices, w.dtype);
@@ -1205,7 +1206,12 @@ extern "C"
 					w.dim[3], invert);
 		MLHIP_CHECK(hipGetLastError());
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_winograd_input_transform(mlContext_t context, int tile_size, const mlTensor_t x, mlTensor_t matrices)
+	try
 	{
 		MLHIP_REQUIRE(x.rank == 4, "Winograd input transform: input must be [B, H, W, C]");
 		require_supported(tile_size, matrices, x.dtype);
@@ -1223,8 +1229,13 @@ extern "C"
 		else
 			launch_input<float>(stream_of(context), x, m);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_winograd_output_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
 			mlTensor_t y, mlActivationType_t act)
+	try
 	{
 		MLHIP_REQUIRE(y.rank == 4, "Winograd output transform: output must be [B, H, W, C]");
 		require_supported(tile_size, matrices, y.dtype);
@@ -1246,8 +1257,13 @@ extern "C"
 		else
 			launch_output<float>(stream_of(context), matrices, bias, ext, out, act);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_winograd_output_input_transform(mlContext_t context, int tile_size, const mlTensor_t matrices, const mlTensor_t bias, const mlTensor_t ext,
 			mlShape_t output_shape, void *output, mlActivationType_t act, mlTensor_t next_matrices)
+	try
 	{
 		MLHIP_REQUIRE(output_shape.rank == 4, "Winograd fused transform: output shape must be [B, H, W, C]");
 		require_supported(tile_size, matrices, matrices.dtype);
@@ -1284,6 +1300,10 @@ extern "C"
 			launch_output_input<half_t, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
 		else
 			launch_output_input<float, 64, 4, 256>(stream_of(context), matrices, bias, ext, output_shape, output, act, next);
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 	static void winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices,
 			mlTensor_t &output_matrices, const mlTensor_t &bias, const mlTensor_t &ext, const mlShape_t &output_shape, void *output, mlActivationType_t act,
@@ -1325,18 +1345,29 @@ extern "C"
 	void hip_winograd_layer_forward(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
 			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
 			mlTensor_t next_matrices)
+	try
 	{
 		winograd_layer_forward(context, tile_size, input_matrices, weight_matrices, output_matrices, bias, ext, output_shape, output, act, next_matrices,
 				false);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_winograd_layer_forward_static(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
 			mlTensor_t output_matrices, const mlTensor_t bias, const mlTensor_t ext, mlShape_t output_shape, void *output, mlActivationType_t act,
 			mlTensor_t next_matrices)
+	try
 	{
 		winograd_layer_forward(context, tile_size, input_matrices, weight_matrices, output_matrices, bias, ext, output_shape, output, act, next_matrices,
 				true);
 	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	int hip_winograd_layer_errors(mlContext_t context)
+	try
 	{
 		MLHIP_CHECK(hipStreamSynchronize(stream_of(context)));
 		unsigned int *word = layer_error_word(get(context)->device_index);
@@ -1345,6 +1376,10 @@ extern "C"
 		if (count != 0)
 			MLHIP_CHECK(hipMemset(word, 0, sizeof(count)));
 		return static_cast<int>(count);
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<int>();
 	}
 } /* extern "C" */
 

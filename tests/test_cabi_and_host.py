@@ -181,3 +181,20 @@ def test_host_side_quantisation_matches_the_oracle():
     transform = Q.symmetric_transform(np.abs(values).max())
     q = Q.quantize_tensor(values, transform)
     assert q.dtype == np.int8 and np.abs(q.astype(np.int32)).max() == 127 and np.abs(q * np.float32(transform[0]) - values).max() <= transform[0] * 0.5001
+
+
+def test_library_errors_surface_as_python_exceptions():
+    """Exceptions cannot unwind through ctypes: the binding switches the library's error capture on, and a failed entry point raises
+    ValueError (std::logic_error: a bad argument) or RuntimeError (std::runtime_error) in Python instead of ending the process. Only
+    argument checks are exercised here: they run before the context or the device is touched."""
+    from minml_amd import backend as B
+
+    desc = B.make_tensor(1, B.DTYPE_FLOAT32, (1, 4, 4, 4))  # never dereferenced: both calls fail on their arguments
+    with pytest.raises(RuntimeError, match="No suitable Winograd transform runtime"):
+        B.fn("winograd_input_transform")(None, 3, desc, B.make_tensor(1, B.DTYPE_FLOAT32, (36, 1, 4)))
+    with pytest.raises(ValueError, match="matrix op"):
+        B.fn("gemm_v2")(None, b"x", b"n", 1.0, desc, desc, 0.0, desc)
+    # the failure was taken: the next call starts clean, and one that succeeds raises nothing
+    assert B.fn("take_last_error")(None, 0) == 0
+    assert B.fn("get_number_of_devices")() >= 0
+    # with capture off the library throws as the reference's backends do (tests/cabi_errors.cpp covers that side from C++)

@@ -83,6 +83,22 @@ def test_gemm_batched_nt_streaming_other_row_lengths(ctx, dtype, K, shape):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_gemm_batched_more_matrices_than_one_grid_dimension_holds(ctx, dtype):
+    """65535 + 5 tiny products in one call (the reference's interface has no limit on the batch); with beta and a broadcast B operand."""
+    rng = np.random.default_rng(11)
+    bt, M, N, K = 65540, 3, 4, 8
+    A = random_tensor(rng, (bt, M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (bt, N, K), dtype, 0.5)
+    C = random_tensor(rng, (bt, M, N), dtype)
+    dC = ml.toDevice(ctx, C)
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), 1.0, 1.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm, beta=1.0, C=C)) <= TOL[dtype]
+    dC.setall(ctx, float("nan"))
+    ml.gemmBatched(ctx, "n", "t", dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm[7]), 1.0, 0.0)
+    assert max_abs_rel(dC.copyToHost(ctx), O.gemm(A, Bm[7])) <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
 def test_gemm_batched_broadcast_and_beta(ctx, dtype):
     rng = np.random.default_rng(5)
     A = random_tensor(rng, (4, 50, 24), dtype)

@@ -86,6 +86,19 @@ def test_global_average_pooling_shapes(ctx, dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
+def test_global_average_pooling_more_images_than_one_grid_dimension_holds(ctx, dtype):
+    shape = (65540, 2, 2, 8)
+    rng = np.random.default_rng(3)
+    x = random_tensor(rng, shape, dtype)
+    y = ml.Tensor((shape[0], shape[3]), dtype)
+    ml.globalAveragePoolingForward(ctx, 1.0, ml.toDevice(ctx, x), 0.0, y)
+    got, want = O.as_float(y.copyToHost(ctx)).astype(np.float64), O.as_float(O.global_average_pooling_forward(x))
+    scale = float(np.abs(O.as_float(x)).mean())
+    assert np.abs(got - want).max() / scale <= TOL[dtype]
+    assert np.abs(got[65535:] - want[65535:]).max() / scale <= TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
 @pytest.mark.parametrize("shape", [(123, 34), (8, 15, 15, 256), (5, 19, 19, 64), (77, 7), (3, 5, 5, 36), (1000, 1), (40, 520)])
 def test_batchnorm_inference_shapes(ctx, dtype, shape):
     """The commented-out reference test uses [123, 34] with TANH (test/backend/test_normalization.cpp:537-568); every activation, the
