@@ -467,7 +467,9 @@ namespace mlhip
 	inline void specialise_epilogue(const FloatEpilogue<T> &e, Launch &&launch)
 	{
 		const bool eligible = e.vectorized && e.bias != nullptr && (e.act == ACTIVATION_RELU || e.act == ACTIVATION_LINEAR);
-		if (!eligible)
+		if (e.vectorized && e.bias == nullptr && e.beta == 0.0f && e.act == ACTIVATION_LINEAR)
+			launch(e.template fixed<ACTIVATION_LINEAR, 0, 0>()); /* the bare product (times alpha) */
+		else if (!eligible)
 			launch(e);
 		else if (e.act == ACTIVATION_RELU)
 		{

@@ -212,9 +212,13 @@ namespace mlhip
 					launch_gemm_dma<half_t>(stream, dma_a, dma_b, g.M, g.N, static_cast<int>(k_bytes), g.batch, g.stride_a * esize, g.stride_b * esize,
 							g.stride_c, ep);
 				else if (fast)
-					hipLaunchKernelGGL((kernel_gemm_nt<half_t, Cfg, FloatEpilogue<half_t>>), fast_grid, dim3(Cfg::THREADS), 0, stream,
-							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
-							g.stride_b, g.stride_c, ep, tiles_n);
+					specialise_epilogue(ep, [&](const auto &fixed)
+					{
+						typedef typename std::decay<decltype(fixed)>::type Fixed;
+						hipLaunchKernelGGL((kernel_gemm_nt<half_t, Cfg, Fixed>), fast_grid, dim3(Cfg::THREADS), 0, stream,
+								reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, static_cast<int>(k_bytes), g.stride_a,
+								g.stride_b, g.stride_c, fixed, tiles_n);
+					});
 				else
 					hipLaunchKernelGGL((kernel_gemm_generic<half_t, float, FloatEpilogue<half_t>>), slow_grid, dim3(256), 0, stream,
 							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,

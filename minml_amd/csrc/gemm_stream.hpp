@@ -495,7 +495,10 @@ namespace mlhip
 	{
 		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
 		constexpr bool WIDE_FITS = PLAIN || KB < 512; /* else B-operand registers + side inputs + a 128-row accumulator exceed 256 VGPRs */
-		if (g.N > 128 && WIDE_FITS)
+		/* slices of 256 columns unless slices of 128 pad N less (N = 384: two wide slices multiply 512 columns, three narrow ones 384;
+		 * measured 252 -> 206 us for the Winograd product at 384 channels) */
+		const bool wide_pads_more = ceil_div(g.N, 256) * 256 > ceil_div(g.N, 128) * 128;
+		if (g.N > 128 && WIDE_FITS && !wide_pads_more)
 		{
 			if constexpr (WIDE_FITS)
 				launch_stream_gemm_as<T, KB, 1, 8>(stream, g, epilogue);
