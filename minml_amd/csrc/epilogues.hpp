@@ -60,6 +60,18 @@ namespace mlhip
 				else
 					return WITH_BIAS != 0;
 			}
+			/* the same epilogue for the columns first .. first + count - 1 only, addressed as columns 0 .. count - 1 */
+			FloatEpilogue columns(int first, int count) const
+			{
+				FloatEpilogue e = *this;
+				e.D += first;
+				if (e.C != nullptr)
+					e.C += first;
+				if (e.bias != nullptr)
+					e.bias += first;
+				e.N = count;
+				return e;
+			}
 			/* the same epilogue with other parts fixed at compile time (the caller guarantees that they agree with the fields) */
 			template<int A, int C, int B>
 			FloatEpilogue<T, A, C, B> fixed() const
@@ -221,6 +233,13 @@ namespace mlhip
 			bool vectorized;
 			static constexpr bool has_c = false;
 
+			Int32Epilogue columns(int first, int count) const
+			{
+				Int32Epilogue e = *this;
+				e.D += first;
+				e.N = count;
+				return e;
+			}
 			struct Column
 			{
 			};
@@ -334,6 +353,17 @@ namespace mlhip
 					return ext != nullptr;
 				else
 					return WITH_EXT != 0;
+			}
+			RequantEpilogue columns(int first, int count) const
+			{
+				RequantEpilogue e = *this;
+				e.D += first;
+				e.scales += first;
+				e.bias += first;
+				if (e.ext != nullptr)
+					e.ext += first;
+				e.N = count;
+				return e;
 			}
 			template<int A, int E>
 			RequantEpilogue<OutT, A, E> fixed() const

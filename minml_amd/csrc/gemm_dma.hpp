@@ -583,7 +583,21 @@ namespace mlhip
 			size_t stride_a_bytes, size_t stride_b_bytes, size_t stride_c, const Epilogue &epilogue)
 	{
 		const int wide = ceil_div(N, 256) * 256, medium = ceil_div(N, 128) * 128, narrow = ceil_div(N, 64) * 64;
-		if (wide <= medium && wide <= narrow)
+		if (N > 256 && N % 256 != 0)
+		{
+			/* e.g. N = 384: the first 256 columns on wide tiles (more flops per operand byte and per fragment read), the remaining
+			 * columns on the tile width that pads them least, instead of narrower tiles throughout */
+			const int first = N / 256 * 256;
+			DenseDmaRows head = b_loader, tail = b_loader;
+			head.rows = first;
+			tail.rows = N - first;
+			tail.base += static_cast<size_t>(first) * (b_loader.row_stride_bytes != 0 ? b_loader.row_stride_bytes : b_loader.k_bytes);
+			launch_gemm_dma_as<T, DmaTileWide>(stream, a_loader, head, M, first, k_bytes, batch, stride_a_bytes, stride_b_bytes, stride_c,
+					epilogue.columns(0, first));
+			launch_gemm_dma<T>(stream, a_loader, tail, M, N - first, k_bytes, batch, stride_a_bytes, stride_b_bytes, stride_c,
+					epilogue.columns(first, N - first));
+		}
+		else if (wide <= medium && wide <= narrow)
 			launch_gemm_dma_as<T, DmaTileWide>(stream, a_loader, b_loader, M, N, k_bytes, batch, stride_a_bytes, stride_b_bytes, stride_c, epilogue);
 		else if (medium <= narrow)
 			launch_gemm_dma_as<T, DmaTileMedium>(stream, a_loader, b_loader, M, N, k_bytes, batch, stride_a_bytes, stride_b_bytes, stride_c, epilogue);

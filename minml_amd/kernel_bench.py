@@ -12,7 +12,8 @@ misc (im2row, element-wise neighbours), heads (softmax, global average pooling, 
 (RMS normalisation and multi-head attention at the hybrid configuration's shape), moe (routing, gather, the two expert layers and
 scatter of that configuration's mixture-of-experts half-block), ceilings (what the chip sustains independent of the
 backend's kernels: read / write / copy streams over buffers that fit the L2s, the 256 MB last-level cache or neither, and a pure MFMA
-loop on constant and on random operands with the shader clock it ran at; needs libminml_ceilings.so, built by minml_amd.build).
+loop on constant and on random operands with the shader clock it ran at; needs libminml_ceilings.so, built by minml_amd.build),
+library (only on request, needs PyTorch: the vendor GEMM library on plain dense products of the convolutions' shapes, as a yardstick).
 """
 import argparse
 import ctypes
@@ -365,12 +366,66 @@ class Bench:
         out8.free()
 
 
+def library(reps):
+    """Yardstick, not part of the backend: what the vendor's GEMM library (hipBLASLt / rocBLAS as PyTorch calls them) reaches on PLAIN dense
+    products of the shapes that the implicit-GEMM convolutions and expert layers reduce to, random operands, no gather, no epilogue.
+    Needs PyTorch; prints a note and returns when it is not importable. Runs in a process that has not loaded the backend library (PyTorch
+    brings a HIP runtime of its own)."""
+    try:
+        import torch
+    except ImportError:
+        print("library   (PyTorch is not importable: no library yardstick)", flush=True)
+        return
+    dev = "cuda"
+    torch.manual_seed(0)
+
+    def row(name, M, N, K, dtype):
+        if dtype == "int8":
+            a = torch.randint(-127, 128, (M, K), dtype=torch.int8, device=dev)
+            b = torch.randint(-127, 128, (K, N), dtype=torch.int8, device=dev)
+            fn = lambda: torch._int_mm(a, b)
+        else:
+            a = torch.randn(M, K, dtype=torch.float16, device=dev)
+            b = torch.randn(N, K, dtype=torch.float16, device=dev) * 0.05
+            fn = lambda: torch.matmul(a, b.t())
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        t = start.elapsed_time(end) / reps * 1e-3
+        ops = 2.0 * M * N * K
+        peak = PEAK[dtype]
+        r = {"group": "library", "kernel": name, "shape": "M=%d N=%d K=%d %s" % (M, N, K, "i8" if dtype == "int8" else "f16"), "us": t * 1e6,
+             "bound": "mfma", "achieved": ops / t / 1e12, "unit": "TOP/s" if dtype == "int8" else "TFLOP/s", "peak": peak / 1e12,
+             "frac": ops / t / peak, "algorithmic_MB": 0.0, "algorithmic_Gop": ops / 1e9}
+        print("%-9s %-34s %-34s %9.1f us  %-4s %9.1f %-7s  %5.1f %%" % ("library", name, r["shape"], r["us"], "mfma", r["achieved"], r["unit"],
+                                                                        100 * r["frac"]), flush=True)
+
+    row("torch.matmul (cfg4 3x3 C=256 as GEMM)", 184832, 256, 2304, "float16")
+    row("torch.matmul (cfg4 5x5 C=256 as GEMM)", 184832, 256, 6400, "float16")
+    row("torch.matmul (cfg4 3x3 C=384 as GEMM)", 184832, 384, 3456, "float16")
+    row("torch.matmul (cfg5 expert layer 1)", 114688, 1024, 256, "float16")
+    row("torch.matmul (cfg5 expert layer 2)", 114688, 256, 1024, "float16")
+    row("torch.matmul (square)", 8192, 8192, 8192, "float16")
+    row("torch._int_mm (cfg3 3x3 C=256 as GEMM)", 230400, 256, 2304, "int8")
+    row("torch._int_mm (square)", 8192, 8192, 8192, "int8")
+
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
+    if args.group == "library":  # only on request: a yardstick that needs PyTorch
+        print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
+        library(args.reps)
+        return 0
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
     for group in ("winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"):
