@@ -91,7 +91,8 @@ namespace
 	 * 1.0 (the pipes toggle little) or pseudo-random halfs / bytes in [-2, 2] (what real data looks like to the multipliers).
 	 * out[0..3] of workgroup 0 = shader-clock ticks and 100 MHz real-time ticks spent in the loop, for the clock the loop ran at.
 	 */
-	template<bool INT8>
+	/* KIND 0: v_mfma_f32_32x32x16_f16, 1: v_mfma_i32_32x32x32_i8, 2: v_mfma_f32_32x32x2_f32 (one float of each operand per lane) */
+	template<int KIND>
 	__global__ __launch_bounds__(256, 1) void kernel_mfma_loop(uint64_t *out, int iters, int random)
 	{
 		const uint32_t lane = threadIdx.x;
@@ -101,8 +102,11 @@ namespace
 			{
 				const uint32_t h = (lane * 2654435761u) ^ ((i * 4 + j) * 40503u) ^ (blockIdx.x * 97u);
 				uint32_t word;
+				constexpr bool INT8 = (KIND == 1);
 				if (INT8)
 					word = random ? (h * 2246822519u) : 0x01010101u;
+				else if (KIND == 2) /* a float with magnitude in [0.5, 1) and a pseudo-random sign, or 1.0 */
+					word = random ? ((0x3f000000u | (h & 0x7fffffu)) ^ ((h << 3) & 0x80000000u)) : 0x3f800000u;
 				else
 				{
 					const uint32_t lo = 0x3000u | (h & 0x8fffu), hi = 0x3000u | ((h >> 16) & 0x8fffu);
@@ -128,7 +132,10 @@ namespace
 #pragma unroll
 				for (int j = 0; j < 4; j++)
 				{
-					if (INT8)
+					if (KIND == 2)
+						accf[i * 4 + j] = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, b[j][0]), __builtin_bit_cast(float, a[i][0]),
+								accf[i * 4 + j], 0, 0, 0);
+					else if (KIND == 1)
 						acci[i * 4 + j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(int4_v, b[j]), __builtin_bit_cast(int4_v, a[i]), acci[i * 4 + j],
 								0, 0, 0);
 					else
@@ -255,13 +262,15 @@ extern "C"
 		check(hipGetLastError(), "launch of kernel_stream");
 	}
 	/* one launch of the MFMA loop on `workgroups` workgroups of 4 wavefronts; `out` = at least 2 + 256 uint64 of device memory */
-	void ceil_mfma(void *stream, void *out, int iters, int random, int int8, int workgroups)
+	void ceil_mfma(void *stream, void *out, int iters, int random, int int8 /* 0 fp16, 1 int8, 2 fp32 */, int workgroups)
 	{
 		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-		if (int8)
-			hipLaunchKernelGGL(kernel_mfma_loop<true>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
+		if (int8 == 1)
+			hipLaunchKernelGGL(kernel_mfma_loop<1>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
+		else if (int8 == 2)
+			hipLaunchKernelGGL(kernel_mfma_loop<2>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
 		else
-			hipLaunchKernelGGL(kernel_mfma_loop<false>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
+			hipLaunchKernelGGL(kernel_mfma_loop<0>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
 		check(hipGetLastError(), "launch of kernel_mfma_loop");
 	}
 }

@@ -350,7 +350,8 @@ class Bench:
         out8 = ml.Tensor((4096,), "uint8")
         iters, wgs = 20000, 256
         for int8, name, peak, ops_per_mfma in ((0, "v_mfma_f32_32x32x16_f16", PEAK["float16"], 2.0 * 32 * 32 * 16),
-                                                (1, "v_mfma_i32_32x32x32_i8", PEAK["int8"], 2.0 * 32 * 32 * 32)):
+                                                (1, "v_mfma_i32_32x32x32_i8", PEAK["int8"], 2.0 * 32 * 32 * 32),
+                                                (2, "v_mfma_f32_32x32x2_f32", PEAK["float32"], 2.0 * 32 * 32 * 2)):
             for random in (0, 1):
                 t = self.time(lambda: lib.ceil_mfma(stream, out8.ptr, iters, random, int8, wgs))
                 ticks = out8.copyToHost(ctx).view(np.uint64)
@@ -358,7 +359,7 @@ class Bench:
                 ops = ops_per_mfma * 16 * iters * 4 * wgs
                 rate = ops / t
                 r = {"group": "ceilings", "kernel": name + " loop", "shape": "%s operands, %d CUs x 4 wavefronts" % ("random" if random else "constant", wgs),
-                     "us": t * 1e6, "bound": "mfma", "achieved": rate / 1e12, "unit": "TOP/s" if int8 else "TFLOP/s", "peak": peak / 1e12,
+                     "us": t * 1e6, "bound": "mfma", "achieved": rate / 1e12, "unit": "TOP/s" if int8 == 1 else "TFLOP/s", "peak": peak / 1e12,
                      "frac": rate / peak, "algorithmic_MB": 0.0, "algorithmic_Gop": ops / 1e9, "shader_clock_GHz": clock_ghz}
                 self.rows.append(r)
                 print("%-9s %-34s %-34s %9.1f us  %-4s %9.1f %-7s  %5.1f %%  shader clock %.2f GHz" % (
