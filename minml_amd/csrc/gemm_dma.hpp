@@ -240,6 +240,23 @@ namespace mlhip
 	 * m = 32*i + l%32 (relative to the wavefront sub-tile). Each wavefront transposes one 32-row slab at a time through its private LDS
 	 * slab [32][WN + 4] and reads it back row-wise, 4 consecutive n per lane, so that the epilogue's global traffic is contiguous along n.
 	 */
+	/*
+	 * The columns of a wavefront's sub-tile that one pass scheme covers: WIDTH / 4 lanes per slab row (4 consecutive n each), hence
+	 * 64 / (WIDTH / 4) rows per pass. Sub-tiles 32, 64 or 128 columns wide are one such part; a 96-column sub-tile is a 64-column part
+	 * followed by a 32-column part.
+	 */
+	template<typename Epilogue, int OFFSET_, int WIDTH_>
+	struct SlabColumns
+	{
+			static constexpr int OFFSET = OFFSET_, WIDTH = WIDTH_;
+			static constexpr int LANES_PER_ROW = WIDTH / 4, ROWS_PER_PASS = 64 / LANES_PER_ROW, PASSES = 32 / ROWS_PER_PASS;
+			static_assert(64 % LANES_PER_ROW == 0 && 32 % ROWS_PER_PASS == 0, "unsupported width of a slab part");
+			int row_in_pass, col, n, n_safe;
+			bool n_valid;
+			typename Epilogue::Column column;
+			typename Epilogue::Extra extra[2][PASSES];
+	};
+
 	template<typename T, typename Cfg, typename Acc, typename Epilogue>
 	__device__ __forceinline__ void store_through_slabs(Acc &acc, uint8_t *lds, int M, int m0, int n0, const Epilogue &epilogue)
 	{
@@ -247,15 +264,8 @@ namespace mlhip
 		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 		const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
 		acc_t *slab = reinterpret_cast<acc_t*>(lds + wave * Cfg::SLAB_BYTES);
-		constexpr int LANES_PER_ROW = Cfg::WN / 4;
-		constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
-		static_assert(64 % LANES_PER_ROW == 0 && 32 % ROWS_PER_PASS == 0, "unsupported wavefront tile width");
 		typedef acc_t vec4 __attribute__((ext_vector_type(4)));
-		constexpr int PASSES = 32 / ROWS_PER_PASS;
-		const int row_in_pass = lane / LANES_PER_ROW;
-		const int col = (lane % LANES_PER_ROW) * 4;
-		const int n = n0 + wave_n * Cfg::WN + col;
-		const int m_base = m0 + wave_m * Cfg::WM + row_in_pass;
+		const int m_wave = m0 + wave_m * Cfg::WM, n_wave = n0 + wave_n * Cfg::WN;
 		auto fill_slab = [&](auto block)
 		{
 			constexpr int i = decltype(block)::value;
@@ -278,6 +288,15 @@ namespace mlhip
 			__builtin_amdgcn_s_waitcnt(0xc07f);
 			__builtin_amdgcn_wave_barrier();
 		};
+		auto place = [&](auto &part)
+		{
+			typedef typename std::decay<decltype(part)>::type Part;
+			part.row_in_pass = lane / Part::LANES_PER_ROW;
+			part.col = Part::OFFSET + (lane % Part::LANES_PER_ROW) * 4;
+			part.n = n_wave + part.col;
+			part.n_valid = part.n < epilogue.N;
+			part.n_safe = part.n_valid ? part.n : 0;
+		};
 		if (epilogue.vectorized)
 		{
 			/*
@@ -285,81 +304,115 @@ namespace mlhip
 			 * epilogue's own loads: the per-column constants are fetched once, and the side inputs (residual) of row block i + 1 are
 			 * requested before row block i is processed, all passes of a block at once, from clamped addresses so that no load
 			 * sits behind a branch.
-			 */
-			const bool n_valid = n < epilogue.N;
-			const int n_safe = n_valid ? n : 0;
-			const typename Epilogue::Column column = epilogue.load_column(n_safe);
-			/*
 			 * A wavefront whose whole sub-tile lies inside the matrix (all but the last row / column tiles) runs the UNCHECKED form:
 			 * no per-pass range test, hence no branch between the side-input loads and their use, so the compiler counts the
 			 * outstanding loads exactly instead of draining them all (vmcnt(0)) in front of every pass.
 			 */
-			const bool inside = __builtin_amdgcn_readfirstlane(
-					static_cast<int>(m0 + wave_m * Cfg::WM + Cfg::WM <= M && n0 + wave_n * Cfg::WN + Cfg::WN <= epilogue.N)) != 0;
-			auto run = [&](auto checked_tag)
+			const bool inside = __builtin_amdgcn_readfirstlane(static_cast<int>(m_wave + Cfg::WM <= M && n_wave + Cfg::WN <= epilogue.N)) != 0;
+			auto run = [&](auto checked_tag, auto &... parts)
 			{
 				constexpr bool CHECKED = decltype(checked_tag)::value;
-				typename Epilogue::Extra extra[2][PASSES];
-				auto request_extras = [&](auto block, auto buffer)
+				auto request_extras = [&](auto &part, auto block, auto buffer)
 				{
+					typedef typename std::decay<decltype(part)>::type Part;
 					constexpr int i = decltype(block)::value, buf = decltype(buffer)::value;
 					if (!epilogue.has_extra())
 						return;
 #pragma unroll
-					for (int pass = 0; pass < PASSES; pass++)
+					for (int pass = 0; pass < Part::PASSES; pass++)
 					{
-						const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
-						extra[buf][pass] = epilogue.load_extra(CHECKED ? min(m, M - 1) : m, n_safe);
+						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
+						part.extra[buf][pass] = epilogue.load_extra(CHECKED ? min(m, M - 1) : m, part.n_safe);
 					}
 				};
-				request_extras(std::integral_constant<int, 0>(), std::integral_constant<int, 0>());
+				auto process = [&](auto &part, auto block)
+				{
+					typedef typename std::decay<decltype(part)>::type Part;
+					constexpr int i = decltype(block)::value;
+#pragma unroll
+					for (int pass = 0; pass < Part::PASSES; pass++)
+					{
+						const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
+						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
+						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
+						if (!CHECKED || (m < M && part.n_valid))
+						{
+							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
+							epilogue.apply(m, part.n, vals, part.column, part.extra[i & 1][pass]);
+						}
+					}
+				};
+				((place(parts), parts.column = epilogue.load_column(parts.n_safe),
+						request_extras(parts, std::integral_constant<int, 0>(), std::integral_constant<int, 0>())), ...);
 				static_for<Cfg::BLOCKS_M>([&](auto block)
 				{
 					constexpr int i = decltype(block)::value;
 					fill_slab(block);
 					if constexpr (i + 1 < Cfg::BLOCKS_M)
-						request_extras(std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>());
-#pragma unroll
-					for (int pass = 0; pass < PASSES; pass++)
-					{
-						const int row = pass * ROWS_PER_PASS + row_in_pass;
-						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + col);
-						const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
-						if (!CHECKED || (m < M && n_valid))
-						{
-							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
-							epilogue.apply(m, n, vals, column, extra[i & 1][pass]);
-						}
-					}
+						(request_extras(parts, std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>()), ...);
+					(process(parts, block), ...);
 					release_slab();
 				});
 			};
-			if (inside)
-				run(std::false_type());
+			if constexpr (Cfg::WN == 96)
+			{
+				SlabColumns<Epilogue, 0, 64> left;
+				SlabColumns<Epilogue, 64, 32> right;
+				if (inside)
+					run(std::false_type(), left, right);
+				else
+					run(std::true_type(), left, right);
+			}
 			else
-				run(std::true_type());
+			{
+				SlabColumns<Epilogue, 0, Cfg::WN> all;
+				if (inside)
+					run(std::false_type(), all);
+				else
+					run(std::true_type(), all);
+			}
 		}
 		else
 		{
 			/* general path: the functor handles ragged and unaligned groups element by element; the passes stay a rolled loop */
-			static_for<Cfg::BLOCKS_M>([&](auto block)
+			auto run = [&](auto &... parts)
 			{
-				constexpr int i = decltype(block)::value;
-				fill_slab(block);
-#pragma clang loop unroll(disable)
-				for (int pass = 0; pass < PASSES; pass++)
+				auto process = [&](auto &part, auto block)
 				{
-					const int row = pass * ROWS_PER_PASS + row_in_pass;
-					const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + col);
-					const int m = m_base + 32 * i + pass * ROWS_PER_PASS;
-					if (m < M)
+					typedef typename std::decay<decltype(part)>::type Part;
+					constexpr int i = decltype(block)::value;
+#pragma clang loop unroll(disable)
+					for (int pass = 0; pass < Part::PASSES; pass++)
 					{
-						acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
-						epilogue(m, n, vals);
+						const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
+						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
+						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
+						if (m < M)
+						{
+							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
+							epilogue(m, part.n, vals);
+						}
 					}
-				}
-				release_slab();
-			});
+				};
+				(place(parts), ...);
+				static_for<Cfg::BLOCKS_M>([&](auto block)
+				{
+					fill_slab(block);
+					(process(parts, block), ...);
+					release_slab();
+				});
+			};
+			if constexpr (Cfg::WN == 96)
+			{
+				SlabColumns<Epilogue, 0, 64> left;
+				SlabColumns<Epilogue, 64, 32> right;
+				run(left, right);
+			}
+			else
+			{
+				SlabColumns<Epilogue, 0, Cfg::WN> all;
+				run(all);
+			}
 		}
 	}
 
@@ -541,6 +594,7 @@ namespace mlhip
 	typedef DmaTileConfig<256, 256, 2, 4, 2, 2, 4> DmaTileWide;
 	typedef DmaTileConfig<256, 128, 4, 2, 2, 2, 2> DmaTileMedium;
 	typedef DmaTileConfig<256, 64, 4, 2, 3, 4, 2> DmaTileNarrow;
+	typedef DmaTileConfig<256, 192, 4, 2, 2, 2, 2> DmaTile192; /* wavefront sub-tiles of 64 x 96: widths that are multiples of 192 but not of 256 (384 channels) */
 
 	/*
 	 * One workgroup per tile; blockIdx.y selects the matrix of a batch (operand bases advance by the given byte strides, D and C of the
@@ -583,7 +637,9 @@ namespace mlhip
 			size_t stride_a_bytes, size_t stride_b_bytes, size_t stride_c, const Epilogue &epilogue)
 	{
 		const int wide = ceil_div(N, 256) * 256, medium = ceil_div(N, 128) * 128, narrow = ceil_div(N, 64) * 64;
-		if (N > 256 && N % 256 != 0)
+		if (N % 192 == 0 && N % 256 != 0)
+			launch_gemm_dma_as<T, DmaTile192>(stream, a_loader, b_loader, M, N, k_bytes, batch, stride_a_bytes, stride_b_bytes, stride_c, epilogue);
+		else if (N > 256 && N % 256 != 0)
 		{
 			/* e.g. N = 384: the first 256 columns on wide tiles (more flops per operand byte and per fragment read), the remaining
 			 * columns on the tile width that pads them least, instead of narrower tiles throughout */
