@@ -161,6 +161,29 @@ def test_gemm_ex_streaming_shapes(ctx, dtype, k_bytes, M, N):
     assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, alpha=1.0, beta=1.0, C=C, act=O.SIGMOID)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "float16"])
+@pytest.mark.parametrize("N", [192, 320, 384, 448, 130, 576])
+def test_gemm_ex_tile_engine_widths(ctx, dtype, N):
+    """K rows of 1024 bytes take the direct-to-LDS tile engine. Its tile width follows N: 256 x 192 tiles for multiples of 192 that are no
+    multiples of 256 (wavefront sub-tiles of 96 columns, whose epilogue walks the slab in two parts), 256 columns on wide tiles plus the
+    rest on a narrower width for 320 / 448, a ragged width (130: the element-wise epilogue), and a ragged last row tile everywhere."""
+    K = 1024 // (2 if dtype == "float16" else 4)
+    M = 1000
+    rng = np.random.default_rng(N)
+    A = random_tensor(rng, (M, K), dtype, 0.3)
+    Bm = random_tensor(rng, (N, K), dtype, 0.3)
+    C = random_tensor(rng, (M, N), dtype)
+    bias = random_tensor(rng, (N,), dtype)
+    dA, dB = ml.toDevice(ctx, A), ml.toDevice(ctx, Bm)
+    dD = ml.Tensor((M, N), dtype)
+    dD.setall(ctx, float("nan"))
+    ml.gemm_ex(ctx, dD, 1.1, "n", dA, "t", dB, 0.5, ml.toDevice(ctx, C), ml.toDevice(ctx, bias), "relu")
+    assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, alpha=1.1, beta=0.5, C=C, bias=bias, act=O.RELU)) <= TOL[dtype]
+    dD.setall(ctx, float("nan"))
+    ml.gemm_ex(ctx, dD, 1.0, "n", dA, "t", dB, 0.0, None, None, "linear")
+    assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm)) <= TOL[dtype]
+
+
 @pytest.mark.parametrize("tag,dtype", [("f32", "float32"), ("f16", "float16")])
 def test_reference_fixtures(ctx, golden, tag, dtype):
     g = golden

@@ -55,7 +55,8 @@ def test_reference_test_case_conv2D_1x1(ctx):
 
 
 @pytest.mark.parametrize("shape,cout,k", [((11, 12, 13, 36), 44, 1), ((3, 12, 13, 32), 44, 5), ((2, 15, 15, 64), 64, 3), ((2, 6, 5, 7), 9, 3),
-                                          ((2, 15, 15, 256), 256, 3), ((1, 19, 19, 48), 20, 3), ((2, 9, 9, 16), 130, 1)])
+                                          ((2, 15, 15, 256), 256, 3), ((1, 19, 19, 48), 20, 3), ((2, 9, 9, 16), 130, 1),
+                                          ((1, 15, 15, 128), 384, 3), ((1, 15, 15, 128), 320, 3)])
 @pytest.mark.parametrize("act", ["relu", "linear"])
 def test_int8_convolution_bit_exact(ctx, shape, cout, k, act):
     """Both device routes — the single fused launch and the reference's three calls (im2row with zero-point padding, int8 GEMM,
