@@ -257,164 +257,171 @@ namespace mlhip
 			typename Epilogue::Extra extra[2][PASSES];
 	};
 
-	template<typename T, typename Cfg, typename Acc, typename Epilogue>
-	__device__ __forceinline__ void store_through_slabs(Acc &acc, uint8_t *lds, int M, int m0, int n0, const Epilogue &epilogue)
+	/*
+	 * The epilogue of a tile in two steps. begin() places the wavefront's lanes on the slab's columns, fetches the per-column constants
+	 * and requests the side inputs (residual) of the first 32-row block; the tile function calls it BEFORE the last chunk of K is
+	 * multiplied (the load queue is empty then: the last chunk's operands have landed and nothing else is requested), so that these
+	 * loads fly under the last chunk's MFMAs instead of at the head of an epilogue that nothing overlaps. finish() transposes the
+	 * accumulators through the slabs and stores. The early requests use clamped addresses (rows past M re-read row M - 1, columns past N
+	 * column 0), so they are valid for edge tiles as well.
+	 */
+	template<typename T, typename Cfg, typename Epilogue>
+	struct SlabEpilogue
 	{
-		typedef typename MfmaTraits<T>::acc_t acc_t;
-		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-		const int wave_m = wave / Cfg::WAVES_N, wave_n = wave % Cfg::WAVES_N;
-		acc_t *slab = reinterpret_cast<acc_t*>(lds + wave * Cfg::SLAB_BYTES);
-		typedef acc_t vec4 __attribute__((ext_vector_type(4)));
-		const int m_wave = m0 + wave_m * Cfg::WM, n_wave = n0 + wave_n * Cfg::WN;
-		auto fill_slab = [&](auto block)
-		{
-			constexpr int i = decltype(block)::value;
+			typedef typename MfmaTraits<T>::acc_t acc_t;
+			typedef acc_t vec4 __attribute__((ext_vector_type(4)));
+			static constexpr bool TWO_PARTS = (Cfg::WN == 96);
+			typedef SlabColumns<Epilogue, 0, TWO_PARTS ? 64 : Cfg::WN> First;
+			typedef SlabColumns<Epilogue, 64, 32> Second;
+			First first;
+			Second second; /* used only by 96-column sub-tiles */
+			int m_wave, n_wave;
+
+			template<typename F>
+			__device__ __forceinline__ void for_parts(F &&f)
+			{
+				f(first);
+				if constexpr (TWO_PARTS)
+					f(second);
+			}
+			template<typename Part, int I, int BUF, bool CLAMP>
+			__device__ __forceinline__ void request_extras(Part &part, const Epilogue &epilogue, int M, std::integral_constant<int, I>, std::integral_constant<int, BUF>,
+					std::integral_constant<bool, CLAMP>)
+			{
+				if (!epilogue.has_extra())
+					return;
 #pragma unroll
-			for (int j = 0; j < Cfg::BLOCKS_N; j++)
-#pragma unroll
-				for (int q = 0; q < 4; q++)
+				for (int pass = 0; pass < Part::PASSES; pass++)
 				{
-					vec4 tmp;
-#pragma unroll
-					for (int e = 0; e < 4; e++)
-						tmp[e] = acc[i][j][q * 4 + e];
-					*reinterpret_cast<vec4*>(slab + (lane & 31) * Cfg::SLAB_STRIDE + 32 * j + 8 * q + 4 * (lane >> 5)) = tmp;
+					const int m = m_wave + part.row_in_pass + 32 * I + pass * Part::ROWS_PER_PASS;
+					part.extra[BUF][pass] = epilogue.load_extra(CLAMP ? min(m, M - 1) : m, part.n_safe);
 				}
-			__builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0): the slab is private to this wavefront, whose LDS operations complete in order */
-			__builtin_amdgcn_wave_barrier();
-		};
-		auto release_slab = [&]()
-		{
-			__builtin_amdgcn_s_waitcnt(0xc07f);
-			__builtin_amdgcn_wave_barrier();
-		};
-		auto place = [&](auto &part)
-		{
-			typedef typename std::decay<decltype(part)>::type Part;
-			part.row_in_pass = lane / Part::LANES_PER_ROW;
-			part.col = Part::OFFSET + (lane % Part::LANES_PER_ROW) * 4;
-			part.n = n_wave + part.col;
-			part.n_valid = part.n < epilogue.N;
-			part.n_safe = part.n_valid ? part.n : 0;
-		};
-		if (epilogue.vectorized)
-		{
-			/*
-			 * Fast path (4-element groups are whole and aligned). A wavefront is alone on its SIMD, so nothing hides the latency of the
-			 * epilogue's own loads: the per-column constants are fetched once, and the side inputs (residual) of row block i + 1 are
-			 * requested before row block i is processed, all passes of a block at once, from clamped addresses so that no load
-			 * sits behind a branch.
-			 * A wavefront whose whole sub-tile lies inside the matrix (all but the last row / column tiles) runs the UNCHECKED form:
-			 * no per-pass range test, hence no branch between the side-input loads and their use, so the compiler counts the
-			 * outstanding loads exactly instead of draining them all (vmcnt(0)) in front of every pass.
-			 */
-			const bool inside = __builtin_amdgcn_readfirstlane(static_cast<int>(m_wave + Cfg::WM <= M && n_wave + Cfg::WN <= epilogue.N)) != 0;
-			auto run = [&](auto checked_tag, auto &... parts)
+			}
+			__device__ __forceinline__ void begin(int M, int m0, int n0, const Epilogue &epilogue)
 			{
-				constexpr bool CHECKED = decltype(checked_tag)::value;
-				auto request_extras = [&](auto &part, auto block, auto buffer)
+				const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+				m_wave = m0 + (wave / Cfg::WAVES_N) * Cfg::WM;
+				n_wave = n0 + (wave % Cfg::WAVES_N) * Cfg::WN;
+				for_parts([&](auto &part)
 				{
 					typedef typename std::decay<decltype(part)>::type Part;
-					constexpr int i = decltype(block)::value, buf = decltype(buffer)::value;
-					if (!epilogue.has_extra())
-						return;
-#pragma unroll
-					for (int pass = 0; pass < Part::PASSES; pass++)
-					{
-						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
-						part.extra[buf][pass] = epilogue.load_extra(CHECKED ? min(m, M - 1) : m, part.n_safe);
-					}
-				};
-				auto process = [&](auto &part, auto block)
-				{
-					typedef typename std::decay<decltype(part)>::type Part;
-					constexpr int i = decltype(block)::value;
-#pragma unroll
-					for (int pass = 0; pass < Part::PASSES; pass++)
-					{
-						const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
-						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
-						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
-						if (!CHECKED || (m < M && part.n_valid))
-						{
-							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
-							epilogue.apply(m, part.n, vals, part.column, part.extra[i & 1][pass]);
-						}
-					}
-				};
-				((place(parts), parts.column = epilogue.load_column(parts.n_safe),
-						request_extras(parts, std::integral_constant<int, 0>(), std::integral_constant<int, 0>())), ...);
-				static_for<Cfg::BLOCKS_M>([&](auto block)
-				{
-					constexpr int i = decltype(block)::value;
-					fill_slab(block);
-					if constexpr (i + 1 < Cfg::BLOCKS_M)
-						(request_extras(parts, std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>()), ...);
-					(process(parts, block), ...);
-					release_slab();
+					part.row_in_pass = lane / Part::LANES_PER_ROW;
+					part.col = Part::OFFSET + (lane % Part::LANES_PER_ROW) * 4;
+					part.n = n_wave + part.col;
+					part.n_valid = part.n < epilogue.N;
+					part.n_safe = part.n_valid ? part.n : 0;
 				});
-			};
-			if constexpr (Cfg::WN == 96)
-			{
-				SlabColumns<Epilogue, 0, 64> left;
-				SlabColumns<Epilogue, 64, 32> right;
-				if (inside)
-					run(std::false_type(), left, right);
-				else
-					run(std::true_type(), left, right);
+				if (epilogue.vectorized)
+					for_parts([&](auto &part)
+					{
+						part.column = epilogue.load_column(part.n_safe);
+						request_extras(part, epilogue, M, std::integral_constant<int, 0>(), std::integral_constant<int, 0>(), std::true_type());
+					});
 			}
-			else
+			template<typename Acc>
+			__device__ __forceinline__ void finish(Acc &acc, uint8_t *lds, int M, const Epilogue &epilogue)
 			{
-				SlabColumns<Epilogue, 0, Cfg::WN> all;
-				if (inside)
-					run(std::false_type(), all);
-				else
-					run(std::true_type(), all);
-			}
-		}
-		else
-		{
-			/* general path: the functor handles ragged and unaligned groups element by element; the passes stay a rolled loop */
-			auto run = [&](auto &... parts)
-			{
-				auto process = [&](auto &part, auto block)
+				const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+				acc_t *slab = reinterpret_cast<acc_t*>(lds + wave * Cfg::SLAB_BYTES);
+				auto fill_slab = [&](auto block)
 				{
-					typedef typename std::decay<decltype(part)>::type Part;
 					constexpr int i = decltype(block)::value;
+#pragma unroll
+					for (int j = 0; j < Cfg::BLOCKS_N; j++)
+#pragma unroll
+						for (int q = 0; q < 4; q++)
+						{
+							vec4 tmp;
+#pragma unroll
+							for (int e = 0; e < 4; e++)
+								tmp[e] = acc[i][j][q * 4 + e];
+							*reinterpret_cast<vec4*>(slab + (lane & 31) * Cfg::SLAB_STRIDE + 32 * j + 8 * q + 4 * (lane >> 5)) = tmp;
+						}
+					__builtin_amdgcn_s_waitcnt(0xc07f); /* lgkmcnt(0): the slab is private to this wavefront, whose LDS operations complete in order */
+					__builtin_amdgcn_wave_barrier();
+				};
+				auto release_slab = [&]()
+				{
+					__builtin_amdgcn_s_waitcnt(0xc07f);
+					__builtin_amdgcn_wave_barrier();
+				};
+				if (epilogue.vectorized)
+				{
+					/*
+					 * Fast path (4-element groups are whole and aligned). A wavefront is alone on its SIMD, so nothing hides the latency of
+					 * the epilogue's own loads: the per-column constants and the first block's side inputs were requested by begin(), and
+					 * the side inputs of row block i + 1 are requested before row block i is processed, all passes of a block at once,
+					 * from clamped addresses so that no load sits behind a branch.
+					 * A wavefront whose whole sub-tile lies inside the matrix (all but the last row / column tiles) runs the UNCHECKED
+					 * form: no per-pass range test, hence no branch between the side-input loads and their use, so the compiler counts
+					 * the outstanding loads exactly instead of draining them all (vmcnt(0)) in front of every pass.
+					 */
+					const bool inside = __builtin_amdgcn_readfirstlane(static_cast<int>(m_wave + Cfg::WM <= M && n_wave + Cfg::WN <= epilogue.N)) != 0;
+					auto run = [&](auto checked_tag)
+					{
+						constexpr bool CHECKED = decltype(checked_tag)::value;
+						static_for<Cfg::BLOCKS_M>([&](auto block)
+						{
+							constexpr int i = decltype(block)::value;
+							fill_slab(block);
+							if constexpr (i + 1 < Cfg::BLOCKS_M)
+								for_parts([&](auto &part)
+								{
+									request_extras(part, epilogue, M, std::integral_constant<int, i + 1>(), std::integral_constant<int, (i + 1) & 1>(),
+											std::integral_constant<bool, CHECKED>());
+								});
+							for_parts([&](auto &part)
+							{
+								typedef typename std::decay<decltype(part)>::type Part;
+#pragma unroll
+								for (int pass = 0; pass < Part::PASSES; pass++)
+								{
+									const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
+									const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
+									const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
+									if (!CHECKED || (m < M && part.n_valid))
+									{
+										acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
+										epilogue.apply(m, part.n, vals, part.column, part.extra[i & 1][pass]);
+									}
+								}
+							});
+							release_slab();
+						});
+					};
+					if (inside)
+						run(std::false_type());
+					else
+						run(std::true_type());
+				}
+				else
+				{
+					/* general path: the functor handles ragged and unaligned groups element by element; the passes stay a rolled loop */
+					static_for<Cfg::BLOCKS_M>([&](auto block)
+					{
+						constexpr int i = decltype(block)::value;
+						fill_slab(block);
+						for_parts([&](auto &part)
+						{
+							typedef typename std::decay<decltype(part)>::type Part;
 #pragma clang loop unroll(disable)
-					for (int pass = 0; pass < Part::PASSES; pass++)
-					{
-						const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
-						const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
-						const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
-						if (m < M)
-						{
-							acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
-							epilogue(m, part.n, vals);
-						}
-					}
-				};
-				(place(parts), ...);
-				static_for<Cfg::BLOCKS_M>([&](auto block)
-				{
-					fill_slab(block);
-					(process(parts, block), ...);
-					release_slab();
-				});
-			};
-			if constexpr (Cfg::WN == 96)
-			{
-				SlabColumns<Epilogue, 0, 64> left;
-				SlabColumns<Epilogue, 64, 32> right;
-				run(left, right);
+							for (int pass = 0; pass < Part::PASSES; pass++)
+							{
+								const int row = pass * Part::ROWS_PER_PASS + part.row_in_pass;
+								const vec4 tmp = *reinterpret_cast<const vec4*>(slab + row * Cfg::SLAB_STRIDE + part.col);
+								const int m = m_wave + part.row_in_pass + 32 * i + pass * Part::ROWS_PER_PASS;
+								if (m < M)
+								{
+									acc_t vals[4] = { tmp[0], tmp[1], tmp[2], tmp[3] };
+									epilogue(m, part.n, vals);
+								}
+							}
+						});
+						release_slab();
+					});
+				}
 			}
-			else
-			{
-				SlabColumns<Epilogue, 0, Cfg::WN> all;
-				run(all);
-			}
-		}
-	}
+	};
 
 	/*
 	 * Computes one BM x BN tile and hands every group of 4 consecutive n of one row m < M to epilogue(m, n, acc[4]) (the functor masks
@@ -548,7 +555,7 @@ namespace mlhip
 			});
 		};
 		constexpr int MFMAS = Cfg::BLOCKS_M * Cfg::BLOCKS_N;
-		for (int c = 0; c < chunks; c++)
+		auto process_chunk = [&](int c) __attribute__((always_inline))
 		{
 			const bool request = (c + DISTANCE < chunks);
 			static_for<KSTEPS>([&](auto kstep)
@@ -581,13 +588,20 @@ namespace mlhip
 				multiply(std::integral_constant<int, HEAD>(), std::integral_constant<int, MFMAS>(), std::integral_constant<int, cur>());
 				__builtin_amdgcn_sched_barrier(0);
 			});
-		}
+		};
+		for (int c = 0; c + 1 < chunks; c++)
+			process_chunk(c);
+		/* the last chunk has been opened with an empty load queue: the epilogue's first loads go out now and land while it is multiplied */
+		SlabEpilogue<T, Cfg, Epilogue> store;
+		store.begin(M, m0, n0, epilogue);
+		if (chunks > 0)
+			process_chunk(chunks - 1);
 
 		/* the slots become the epilogue's slabs: every wavefront must have finished reading fragments */
 		__builtin_amdgcn_s_waitcnt(0xc07f);
 		barrier_no_fence();
 
-		store_through_slabs<T, Cfg>(acc, lds, M, m0, n0, epilogue);
+		store.finish(acc, lds, M, epilogue);
 	}
 
 	/* tile shapes by output width: wavefront sub-tiles of 128x128, 128x64 and 64x64 */
