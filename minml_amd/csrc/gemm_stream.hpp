@@ -435,15 +435,19 @@ namespace mlhip
 			int M, N, k_bytes, batch;
 			size_t stride_a, stride_b, stride_c;
 	};
-	/* enough 128-row units to give every CU several, and a K row length the kernel is instantiated for */
+	/*
+	 * A K row length the kernel is instantiated for. There is no lower bound on the size of the product: with a single unit per
+	 * workgroup the kernel still starts faster than the tile engine (its B operand goes straight to registers and its first stage is one
+	 * 16 KB request), e.g. 10 against 19 us for the 36 products of one 15x15 position.
+	 */
 	inline bool stream_gemm_applies(int M, int batch, size_t k_bytes)
 	{
-		return (k_bytes == 128 || k_bytes == 256 || k_bytes == 512) && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256;
+		return (k_bytes == 128 || k_bytes == 256 || k_bytes == 512) && M > 0 && batch > 0;
 	}
 	/* the fp16 forms are also instantiated for 768-byte rows (384 halfs), whose B operand still fits the registers */
 	inline bool stream_gemm_half_applies(int M, int batch, size_t k_bytes)
 	{
-		return stream_gemm_applies(M, batch, k_bytes) || (k_bytes == 768 && static_cast<size_t>(batch) * ceil_div(M, 128) >= 256);
+		return stream_gemm_applies(M, batch, k_bytes) || (k_bytes == 768 && M > 0 && batch > 0);
 	}
 	inline bool stream_gemm_plain_applies(int M, int batch, size_t k_bytes, int element_size)
 	{
