@@ -6,7 +6,7 @@ implementation must move (inputs once, outputs once) and the flops / integer ops
 the two takes longer at the chip's peaks (HBM 8 TB/s; dense MFMA fp16 2.5 PFLOP/s, int8 5.0 POP/s, fp32 157.3 TFLOP/s); `frac` is the
 achieved fraction of that peak.
 
-Groups: winograd (transforms and batched GEMM at the residual-network shapes), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
+Groups: winograd (transforms and batched GEMM at the residual-network shapes), small (the same launches at 1 to 128 positions), conv (implicit-GEMM sweep: 19x19 boards, batch 512,
 channels 64..384, kernels 1 / 3 / 5, bias + residual + ReLU), int8 (quantised 3x3 convolution at 256 channels and its three-call form),
 misc (im2row, element-wise neighbours), heads (softmax, global average pooling, batch normalisation in inference mode), transformer
 (RMS normalisation and multi-head attention at the hybrid configuration's shape), moe (routing, gather, the two expert layers and
@@ -117,6 +117,38 @@ class Bench:
                 V2.free()
             for t in (x, y, w, bias, U, V, M):
                 t.free()
+
+    def small(self):
+        """The launches of one residual block of the 20 x 256 network at small batches (1, 8, 32, 128 positions): there the time of a launch is
+        its start-up and one pass through its pipeline, not bandwidth or arithmetic; 'of peak' is shown for completeness only."""
+        ctx, rng = self.ctx, self.rng
+        board, chans, dtype, s = 15, 256, "float16", 2
+        wshape = (chans, 3, 3, chans)
+        w = _random(ctx, wshape, dtype, rng, 0.05)
+        bias = _random(ctx, (chans,), dtype, rng, 0.1)
+        U = ml.Tensor((36, chans, chans), dtype)
+        ml.winogradWeightTransform(ctx, w, U)
+        for batch in (1, 8, 32, 128):
+            tiles, pix = batch * 16, batch * board * board
+            x = _random(ctx, (batch, board, board, chans), dtype, rng)
+            y = ml.Tensor((batch, board, board, chans), dtype)
+            V = ml.Tensor((36, tiles, chans), dtype)
+            M = ml.Tensor((36, tiles, chans), dtype)
+            V2 = ml.Tensor((36, tiles, chans), dtype)
+            M.zeroall(ctx)
+            shape = "cfg2 layer at B=%d 15x15 C=256 f16" % batch
+            oshape = (batch, board, board, chans)
+            self.row("small", "winograd_input_transform", shape, lambda: ml.winogradInputTransform(ctx, wshape, x, V), s * (pix * chans + 36 * tiles * chans))
+            self.row("small", "gemm_batched (36 x T x C x C)", shape, lambda: ml.gemmBatched(ctx, "n", "t", M, V, U, 1.0, 0.0),
+                     s * 36 * (2 * tiles * chans + chans * chans), 2.0 * 36 * tiles * chans * chans, dtype)
+            self.row("small", "winograd_output_input_transform", shape,
+                     lambda: ml.winogradOutputInputTransform(ctx, wshape, M, oshape, None, bias, None, "relu", V2), s * 2 * 36 * tiles * chans)
+            self.row("small", "winograd_output_transform +res", shape, lambda: ml.winogradOutputTransform(ctx, wshape, M, y, bias, x, "relu"),
+                     s * (36 * tiles * chans + 2 * pix * chans + chans))
+            for t in (x, y, V, M, V2):
+                t.free()
+        for t in (w, bias, U):
+            t.free()
 
     def conv(self):
         ctx, rng = self.ctx, self.rng
@@ -419,7 +451,7 @@ def library(reps):
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
@@ -429,7 +461,7 @@ def main():
         return 0
     bench = Bench(args.reps)
     print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
-    for group in ("winograd", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"):
+    for group in ("winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings"):
         if args.group in ("all", group):
             getattr(bench, group)()
     if args.json:
