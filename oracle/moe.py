@@ -1,14 +1,24 @@
 """CPU statement of the mixture-of-experts steps (routing, gather, expert layers, scatter). TEST INFRASTRUCTURE ONLY.
 
-PARITY UNPINNED against the reference: its core dispatches these operations to the CUDA backend only (src/core/math.cpp:1328-1491 does
-nothing on the CPU), so no CPU result of the reference exists to compare with. The functions below state what the reference's device
-kernels compute (src/backend/cuda/kernels/moe.cu; lines cited per function) in plain numpy, with the two freedoms those kernels leave
-fixed as follows: (1) ties — the reference's bitonic sorts order equal scores by the sorting network, here equal scores are ordered by
-ascending token index; (2) accumulation — the reference scatters with atomic additions in the storage type (arrival order, one rounding
-per addition), here contributions are summed in fp32 in ascending expert order and rounded once. fp16 results are stored by truncation
-like everything else in this backend's CPU counterpart (src/backend/cpu/fp16.hpp:61-68). What pins these functions instead is in
-tests/test_oracle_pins.py: top-k against a brute-force search, permutation equivariance, gather / scatter against index arithmetic written
-independently, scatter(gather(x)) = x * (sum of gates per token), the expert layers against one dense product per expert.
+The reference's core dispatches these operations to the CUDA backend only (src/core/math.cpp:1328-1491 does nothing on the CPU), so no
+CPU result of the reference's library exists to compare with. What the reference does hold is its own test file,
+test/backend/test_moe.cpp, whose CPU baselines its device layers are tested against (difference at most 1e-4 in fp32). The functions
+below state what the reference's device kernels compute (src/backend/cuda/kernels/moe.cu; lines cited per function) in plain numpy, and
+are pinned as follows (tests/test_oracle_moe.py; the baselines are restated in tests/reference_moe_baselines.py):
+  * gather_tokens, scatter_tokens, hash_routing, token_choice_routing (without bias), moe_forward, get_capacity: against those
+    baselines at the shapes of the reference's tests - gather and hash exactly, scatter bit for bit (same additions, same order),
+    the routed tokens and slots exactly and the gates to 1e-6, the expert layers within the reference test's own 1e-4;
+  * expert_choice_routing: PARITY UNPINNED against the reference. The baseline's branch for it (test_moe.cpp:547-566) is nested
+    inside the token-choice branch and never runs, and it computes a softmax over the selected scores where the device kernel
+    applies a sigmoid (moe.cu:438-479); the function follows the kernel and is pinned by what the mathematics fixes: the top-k
+    against a brute-force search, permutation equivariance, gate = sigmoid of the selected score;
+  * the bias of token_choice_routing (the baseline has none) and beta != 0 in gather / scatter: by the kernels' text and by
+    identities (scatter(gather(x)) = x * (sum of gates per token), beta-linearity).
+Two freedoms that the reference's kernels leave are fixed here: (1) ties - the reference's bitonic sorts (and its baseline's std::sort)
+order equal scores arbitrarily, here equal scores are ordered by ascending token index; (2) accumulation - the reference scatters with
+atomic additions in the storage type (arrival order, one rounding per addition), here contributions are summed in fp32 in ascending
+expert order (the order of the reference test's baseline) and rounded once. fp16 results are stored by truncation like everything
+else in this backend's CPU counterpart (src/backend/cpu/fp16.hpp:61-68).
 
 Tensors: scores [B, H, W, E]; indices_and_values [B, 2, E, K] in the storage type (plane 0: token indices as numbers, -1 for an empty
 slot; plane 1: gate values); gathered tokens [B, K, E, C]; expert weights [E, N, C], bias [E, N].

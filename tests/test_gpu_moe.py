@@ -128,3 +128,67 @@ def test_expert_layers(ctx, dtype, dims):
     dy = ml.toDevice(ctx, y0)
     ml.moeForward(ctx, dx, dw, db, 0.5, dy, "linear")
     assert max_abs_rel(dy.copyToHost(ctx), M.moe_forward(x, w, bias, O.LINEAR, beta=0.5, y=y0)) <= TOL[dtype]
+
+
+# ---- the reference's own tests, mirrored: its device layers against the CPU baselines of test/backend/test_moe.cpp, fp32, 1e-4 -----------
+
+def _routing_table(rng, batch, tokens, experts, slots, empty=0.15):
+    table = np.zeros((batch, 2, experts, slots), np.float32)
+    for b in range(batch):
+        for e in range(experts):
+            table[b, 0, e] = rng.permutation(tokens)[:slots]
+    table[:, 1] = rng.random((batch, experts, slots), dtype=np.float32)
+    table[:, 0][rng.random((batch, experts, slots)) < empty] = -1.0
+    return table
+
+
+def test_reference_test_router_token_choice_and_hash(ctx):
+    """TestRouter (test_moe.cpp:956-981): token choice with capacity factor 1.25 on [128, 15, 15, 2] in fp32 against the test's
+    BaselineRouter, difference at most 1e-4; and the baseline's hash branch."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(31)
+    shape = (128, 15, 15, 2)
+    scores = rng.standard_normal(shape, dtype=np.float32)
+    cap = R.capacity(1.25, 225, 2)
+    iv = ml.Tensor((128, 2, 2, cap), "float32")
+    ml.tokenChoiceRoutingForward(ctx, ml.toDevice(ctx, scores), None, iv)
+    got, want = iv.copyToHost(ctx), R.token_choice_router(scores, cap)
+    assert np.array_equal(got[:, 0], want[:, 0])
+    assert np.abs(got[:, 1] - want[:, 1]).max() <= 1e-4
+    ml.hashRouting(ctx, ml.toDevice(ctx, scores), iv)
+    assert np.array_equal(iv.copyToHost(ctx), R.hash_router(128, 225, 2, cap))
+
+
+def test_reference_test_gather_and_scatter(ctx):
+    """TestGatherTopK / TestScatterTopK (test_moe.cpp:989-1056): [3, 11, 12, 56], 8 experts, 12 and 16 slots, fp32, against the test's
+    baselines; gather is a copy (exact), scatter within 1e-4."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(32)
+    x = rng.standard_normal((3, 11, 12, 56), dtype=np.float32)
+    table = _routing_table(rng, 3, 132, 8, 12)
+    y = ml.Tensor((3, 12, 8, 56), "float32")
+    y.setall(ctx, float("nan"))
+    ml.gatherTokensForward(ctx, ml.toDevice(ctx, x), ml.toDevice(ctx, table), 0.0, y)
+    assert np.array_equal(y.copyToHost(ctx), R.gather_tokens(x, table))
+    rows = rng.standard_normal((3, 16, 8, 56), dtype=np.float32)
+    table = _routing_table(rng, 3, 132, 8, 16)
+    out = ml.Tensor((3, 11, 12, 56), "float32")
+    out.setall(ctx, float("nan"))
+    ml.scatterTokensForward(ctx, ml.toDevice(ctx, rows), ml.toDevice(ctx, table), 0.0, out)
+    want = R.scatter_tokens(rows, table, (3, 11, 12, 56))
+    assert np.abs(out.copyToHost(ctx) - want).max() / np.abs(want).max() <= 1e-4
+
+
+@pytest.mark.parametrize("act", ["relu", "linear"])
+def test_reference_test_mixture_of_experts(ctx, act):
+    """TestMixtureOfExperts (test_moe.cpp:1067-1093): [32, 16, 32, 128] -> 64 neurons per expert in fp32 against the test's baseline
+    (a plain triple loop per expert, then bias and activation), difference at most 1e-4."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(33)
+    x = rng.standard_normal((32, 16, 32, 128), dtype=np.float32)
+    w = rng.standard_normal((32, 64, 128), dtype=np.float32) * np.float32(0.1)
+    b = rng.standard_normal((32, 64), dtype=np.float32) * np.float32(0.1)
+    y = ml.Tensor((32, 16, 32, 64), "float32")
+    ml.moeForward(ctx, ml.toDevice(ctx, x), ml.toDevice(ctx, w), ml.toDevice(ctx, b), 0.0, y, act)
+    want = R.expert_layers(x, w, b, act == "relu")
+    assert np.abs(y.copyToHost(ctx) - want).max() / np.abs(want).max() <= 1e-4

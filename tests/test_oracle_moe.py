@@ -144,3 +144,67 @@ def test_expert_layers_are_one_dense_product_per_expert(dtype):
     w2[1] = conv(rng.standard_normal((n, c)))
     y2 = M.moe_forward(x, w2, bias, O.RELU)
     assert np.array_equal(np.asarray(y2)[:, :, 0], np.asarray(M.moe_forward(x, w, bias, O.RELU))[:, :, 0])
+
+
+# ---- the reference's own test baselines (test/backend/test_moe.cpp), at the shapes its tests use ---------------------------------------
+
+def _table(rng, batch, tokens, experts, slots, empty=0.15):
+    """A routing table with distinct tokens per expert row, random gates and some empty (-1) slots."""
+    table = np.zeros((batch, 2, experts, slots), np.float32)
+    for b in range(batch):
+        for e in range(experts):
+            table[b, 0, e] = rng.permutation(tokens)[:slots]
+    table[:, 1] = rng.random((batch, experts, slots), dtype=np.float32)
+    hole = rng.random((batch, experts, slots)) < empty
+    table[:, 0][hole] = -1.0
+    return table
+
+
+def test_gather_equals_the_reference_tests_baseline():
+    """TestGatherTopK: [3, 11, 12, 56], 8 experts, 12 slots (test_moe.cpp:989-1000)."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(21)
+    x = rng.standard_normal((3, 11, 12, 56), dtype=np.float32)
+    table = _table(rng, 3, 11 * 12, 8, 12)
+    assert np.array_equal(M.gather_tokens(x, table), R.gather_tokens(x, table))
+
+
+def test_scatter_equals_the_reference_tests_baseline():
+    """TestScatterTopK: [3, 16, 8, 56] back to [3, 11, 12, 56] (test_moe.cpp:1028-1039). Same additions in the same order: equal bits."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(22)
+    x = rng.standard_normal((3, 16, 8, 56), dtype=np.float32)
+    table = _table(rng, 3, 11 * 12, 8, 16)
+    assert np.array_equal(M.scatter_tokens(x, table, (3, 11, 12, 56)), R.scatter_tokens(x, table, (3, 11, 12, 56)))
+
+
+def test_hash_and_token_choice_routing_equal_the_reference_tests_baseline():
+    """TestRouter: token choice with capacity factor 1.25 on [128, 15, 15, 2] (test_moe.cpp:956-981; a smaller batch here), and the
+    baseline's hash branch. Tokens and slots must agree exactly (random fp32 scores have no equal probabilities), gates to rounding:
+    the baseline shifts the softmax by the row maximum, the device kernel that the oracle follows by the maximum of score + bias."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(23)
+    scores = rng.standard_normal((16, 15, 15, 2), dtype=np.float32)
+    cap = R.capacity(1.25, 225, 2)
+    assert cap == M.get_capacity(1.25, 225, 2) == 140
+    want = R.token_choice_router(scores, cap)
+    got = M.token_choice_routing(scores, None, cap)
+    assert np.array_equal(got[:, 0], want[:, 0])
+    assert np.abs(got[:, 1] - want[:, 1]).max() <= 1e-6
+    for experts in (2, 8, 7):
+        cap = R.capacity(1.25, 225, experts)
+        assert np.array_equal(M.hash_routing(np.zeros((3, 15, 15, experts), np.float32), cap), R.hash_router(3, 225, experts, cap))
+
+
+def test_expert_layers_equal_the_reference_tests_baseline():
+    """TestMixtureOfExperts: [32, 16, 32, 128] -> 64 neurons (test_moe.cpp:1067-1093; a smaller batch here), within the reference
+    test's own bound of 1e-4 (the baseline sums a row's products one by one, the oracle in the order of the reference's GEMM)."""
+    import reference_moe_baselines as R
+    rng = np.random.default_rng(24)
+    x = rng.standard_normal((4, 16, 32, 128), dtype=np.float32)
+    w = (rng.standard_normal((32, 64, 128), dtype=np.float32) * np.float32(0.1))
+    b = rng.standard_normal((32, 64), dtype=np.float32) * np.float32(0.1)
+    for relu in (True, False):
+        got = M.moe_forward(x, w, b, O.RELU if relu else O.LINEAR)
+        want = R.expert_layers(x, w, b, relu)
+        assert np.abs(got - want).max() / np.abs(want).max() <= 1e-4
