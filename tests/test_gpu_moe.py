@@ -1,5 +1,5 @@
 """Mixture-of-experts steps on the GPU against their CPU statement (oracle/moe.py; the reference has no CPU implementation of these,
-so that statement is pinned by tests/test_oracle_moe.py instead), through the C-ABI: routing tables must agree in every index (scores
+so that statement is pinned by tests/test_oracle_moe.py against the baselines of the reference's own tests instead), through the C-ABI: routing tables must agree in every index (scores
 are drawn so that no two tokens tie) and in the gates to rounding; gather is an exact copy; expert layers and scatter within the GEMM
 tolerances (fp32 1e-4, fp16 1e-2 max-abs relative)."""
 import numpy as np
