@@ -40,7 +40,8 @@ def test_against_reference_fixtures(ctx, golden):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
-@pytest.mark.parametrize("shape", [(230, 256), (64, 15, 15, 64), (7, 100), (5, 33), (3, 1), (9, 1024), (4, 2056), (1000, 8)])
+@pytest.mark.parametrize("shape", [(230, 256), (64, 15, 15, 64), (7, 100), (5, 33), (3, 1), (9, 1024), (4, 2056), (1000, 8),
+                                   (123, 43)])  # the last: the reference's own test (test/backend/test_normalization.cpp:977-986)
 def test_rmsnorm_shapes(ctx, dtype, shape):
     rng = np.random.default_rng(sum(shape))
     x, gamma = random_tensor(rng, shape, dtype, 2.0), random_tensor(rng, shape[-1:], dtype)
@@ -73,6 +74,7 @@ def test_rmsnorm_in_place_and_zero_rows(ctx):
     (2, 15, 15, 4, 32, 8, True),     # symmetric layout: k = q
     (2, 6, 5, 3, 24, 3, False),      # heads of 24: the plain kernel
     (1, 20, 20, 2, 16, 0, True),     # heads of 16, 400 tokens: the plain kernel
+    (3, 13, 14, 4, 14, 14, False),   # the reference's own test: 56 channels in 4 heads, table range max(13, 14) (test/backend/test_attention.cpp:441-451)
 ])
 def test_attention_shapes(ctx, dtype, case):
     b, h, w, heads, d, r, symmetric = case
