@@ -334,6 +334,26 @@ def test_elementwise_neighbours(ctx, dtype):
     assert max_abs_rel(dy.copyToHost(ctx), O.add_tensors(y0, 0.5, x, -2.0, x, 0.0, None, 0.25)) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype,limit", [("float32", 1e-6), ("float16", 1e-3)])
+def test_reference_tests_of_the_elementwise_neighbours(ctx, dtype, limit):
+    """The reference's own tests, at their shapes and limits (test/backend/test_tensor_op.cpp:293-350, 408-435): addBiasAct in place with a
+    sigmoid on [123, 48] (mean absolute difference at most 1e-6 in fp32, 1e-3 in fp16), addTensors of two [123, 14] tensors (1e-6)."""
+    rng = np.random.default_rng(48)
+    x = random_tensor(rng, (123, 48), dtype)
+    b = random_tensor(rng, (48,), dtype)
+    dy = ml.toDevice(ctx, x)
+    ml.addBiasAct(ctx, 1.0, dy, ml.toDevice(ctx, b), 0.0, dy, "sigmoid")
+    xf, bf = O.as_float(x).astype(np.float64), O.as_float(b).astype(np.float64)
+    baseline = 1.0 / (1.0 + np.exp(-(xf + bf[None, :])))
+    assert np.abs(O.as_float(dy.copyToHost(ctx)) - baseline).mean() <= limit
+    if dtype == "float32":
+        s1, s2 = random_tensor(rng, (123, 14), dtype), random_tensor(rng, (123, 14), dtype)
+        dst = ml.Tensor((123, 14), dtype)
+        dst.zeroall(ctx)
+        ml.addTensors(ctx, 1.0, ml.toDevice(ctx, s1), 1.0, ml.toDevice(ctx, s2), 0.0, None, 0.0, dst)
+        assert np.abs(dst.copyToHost(ctx).astype(np.float64) - (s1.astype(np.float64) + s2)).mean() <= 1e-6
+
+
 def test_convert_and_unpack(ctx, golden):
     g = golden
     src = g["cvt_src"]
