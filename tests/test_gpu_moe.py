@@ -82,7 +82,9 @@ def test_hash_routing(ctx):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
-@pytest.mark.parametrize("shape,experts,capacity", [((2, 15, 15, 256), 8, 56), ((2, 5, 7, 12), 3, 40), ((1, 4, 4, 7), 2, 5)])
+@pytest.mark.parametrize("shape,experts,capacity", [((2, 15, 15, 256), 8, 56), ((2, 5, 7, 12), 3, 40), ((1, 4, 4, 7), 2, 5),
+                                                    ((2, 6, 6, 16), 12, 5),      # more experts than one group of eight
+                                                    ((1, 19, 19, 8), 40, 12)])   # inverted table too large for LDS: the scanning form
 def test_gather_and_scatter(ctx, dtype, shape, experts, capacity):
     rng = np.random.default_rng(sum(shape))
     b, h, w, c = shape
