@@ -38,6 +38,7 @@ namespace mlhip
 			bool vectorized; /* N % 4 == 0 and D, C, bias 4-element aligned */
 			int bias_batch_stride = 0; /* elements between the biases of consecutive matrices of a batch (0: one bias for all) */
 			static constexpr bool has_c = true;
+			static constexpr bool no_side_input = (WITH_C == 0); /* known at compile time: nothing is read per output element */
 
 			__device__ __forceinline__ int activation() const
 			{
@@ -138,6 +139,24 @@ namespace mlhip
 				x.raw = *reinterpret_cast<const decltype(x.raw)*>(C + static_cast<size_t>(m) * row_stride + n);
 				return x;
 			}
+			/* only when nothing is read per element (no_side_input): the 4 finished results, same arithmetic and order as apply() */
+			__device__ __forceinline__ Vec<T, 4> value(const float (&acc)[4], const Column &col) const
+			{
+				Vec<T, 4> out;
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					out.v[e] = acc[e] * alpha;
+				if (with_bias())
+				{
+#pragma unroll
+					for (int e = 0; e < 4; e++)
+						out.v[e] += col.bias[e];
+				}
+#pragma unroll
+				for (int e = 0; e < 4; e++)
+					out.v[e] = finish(out.v[e]);
+				return out;
+			}
 			__device__ __forceinline__ void apply(int m, int n, const float (&acc)[4], const Column &col, const Extra &x) const
 			{
 				Vec<T, 4> out;
@@ -232,6 +251,7 @@ namespace mlhip
 			int row_stride;
 			bool vectorized;
 			static constexpr bool has_c = false;
+			static constexpr bool no_side_input = false;
 
 			Int32Epilogue columns(int first, int count) const
 			{
@@ -352,6 +372,7 @@ namespace mlhip
 			int act;
 			bool vectorized; /* N % 4 == 0 and all pointers 4-element aligned */
 			static constexpr bool has_c = false;
+			static constexpr bool no_side_input = false;
 
 			__device__ __forceinline__ int activation() const
 			{

@@ -23,6 +23,7 @@
 
 #include "common.hpp"
 #include "gemm_core.hpp"
+#include "epilogues.hpp"
 
 #include <type_traits>
 
@@ -105,6 +106,18 @@ namespace mlhip
 	struct PlainStore
 	{
 	};
+	/* epilogues that read nothing per output element (PlainStore; functors whose residual is absent at compile time): their results are
+	 * finished in the accumulator registers and cross the slab in the output type, 16 bytes per lane on the way out */
+	template<typename Epilogue>
+	struct stream_epilogue_reads_nothing
+	{
+			static constexpr bool value = Epilogue::no_side_input;
+	};
+	template<>
+	struct stream_epilogue_reads_nothing<PlainStore>
+	{
+			static constexpr bool value = true;
+	};
 
 	/*
 	 * One workgroup of WAVES_M x WAVES_N wavefronts covers a unit of 128 rows x 32 * WAVES_N columns; a wavefront owns 128 / WAVES_M
@@ -115,13 +128,14 @@ namespace mlhip
 	 */
 	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue>
 	__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a,
-			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, int sweep, Epilogue epilogue)
+			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, int sweep, size_t a_row_bytes, Epilogue epilogue)
 	{
 		typedef StreamGemmConfig Cfg;
 		typedef MfmaTraits<T> Traits;
 		typedef typename Traits::acc_vec acc_vec;
 		typedef typename Traits::acc_t acc_t;
 		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
+		constexpr bool PACKED = stream_epilogue_reads_nothing<Epilogue>::value;
 		constexpr int WAVES = WAVES_M * WAVES_N;
 		constexpr int BN = 32 * WAVES_N;
 		constexpr int ROWS = Cfg::BM / WAVES_M; /* rows of a unit owned by one wavefront */
@@ -129,7 +143,7 @@ namespace mlhip
 		constexpr int STAGES_PER_UNIT = KB / Cfg::STAGE_K_BYTES;
 		constexpr int DISTANCE = STAGES - 1; /* stages requested ahead of the one being multiplied */
 		constexpr int LOADS = 16 / WAVES; /* 1 KB blocks of a 16 KB stage moved by one wavefront */
-		constexpr int SLAB_STRIDE = 32 * (PLAIN ? sizeof(T) : 4) + 16;
+		constexpr int SLAB_STRIDE = 32 * (PACKED ? sizeof(T) : 4) + 16;
 		constexpr int KSTEPS = 4; /* MFMA k steps per stage */
 		static_assert(KB % Cfg::STAGE_K_BYTES == 0 && ROWS % 32 == 0, "unsupported unit shape");
 		static_assert(16 % WAVES == 0 && DISTANCE >= 2 && DISTANCE <= 8 && (DISTANCE - 2) * LOADS <= 63, "unsupported workgroup shape");
@@ -205,7 +219,11 @@ namespace mlhip
 			{
 				local.D += static_cast<size_t>(matrix) * stride_c;
 				if constexpr (Epilogue::has_c)
+				{
 					local.C += static_cast<size_t>(matrix) * stride_c;
+					if (local.bias != nullptr)
+						local.bias += static_cast<size_t>(matrix) * local.bias_batch_stride; /* 0 unless every matrix has its own bias */
+				}
 			}
 
 			wait_vmcnt<0>();
@@ -229,7 +247,7 @@ namespace mlhip
 				for (int i = 0; i < LOADS; i++)
 				{
 					const int m = min(m_first + load_row[i], M - 1); /* rows past the end re-read the last row; their products are never stored */
-					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * KB + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
+					__builtin_amdgcn_global_load_lds((global_ptr_t) (a_base + static_cast<size_t>(m) * a_row_bytes + ks * Cfg::STAGE_K_BYTES + load_chunk_bytes[i]),
 							(lds_ptr_t) (stage + (wave + WAVES * i) * 1024), 16, 0, 2); /* non-temporal: every row of A is read once */
 				}
 			};
@@ -285,14 +303,40 @@ namespace mlhip
 							side.extra[i][pass] = local.load_extra(min(m_first + 32 * i + pass * 8 + (lane >> 3), M - 1), side_n);
 				}
 			};
-			if constexpr (!PLAIN)
+			if constexpr (!PACKED)
 				side.column = local.load_column(side_n);
+			/* packed form: the constants of this lane's 4 consecutive n in each of the 4 register groups of an accumulator block */
+			typename std::conditional<PLAIN, NoSide, Epilogue>::type::Column packed_columns[4];
+			if constexpr (PACKED && !PLAIN)
+			{
+#pragma unroll
+				for (int q = 0; q < 4; q++)
+				{
+					const int n = n0 + 8 * q + 4 * half_sel;
+					packed_columns[q] = local.load_column(n < local.N ? n : 0);
+				}
+			}
 			auto store_unit = [&](int u) __attribute__((always_inline))
 			{
 				/* lane l, register r of block i: m = 32 i + l % 32, n = 8 (r / 4) + 4 (l / 32) + r % 4 */
 				const int m_first = (tile_base + u * tile_step) * Cfg::BM + wave_m * ROWS;
-				if constexpr (PLAIN)
+				if constexpr (PACKED)
 				{
+					T *out_base;
+					size_t out_stride;
+					int out_n;
+					if constexpr (PLAIN)
+					{
+						out_base = c_base;
+						out_stride = N;
+						out_n = N;
+					}
+					else
+					{
+						out_base = local.D;
+						out_stride = local.row_stride;
+						out_n = local.N;
+					}
 					constexpr int ELEMS_PER_16B = 16 / sizeof(T);
 					constexpr int LANES_PER_ROW = 32 / ELEMS_PER_16B;
 					constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
@@ -304,9 +348,17 @@ namespace mlhip
 						for (int q = 0; q < 4; q++)
 						{
 							Vec<T, 4> v;
+							if constexpr (PLAIN)
+							{
 #pragma unroll
-							for (int e = 0; e < 4; e++)
-								v.v[e] = acc[i][4 * q + e];
+								for (int e = 0; e < 4; e++)
+									v.v[e] = acc[i][4 * q + e];
+							}
+							else
+							{
+								const acc_t vals[4] = { acc[i][4 * q + 0], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3] };
+								v = local.value(vals, packed_columns[q]);
+							}
 							v.store(reinterpret_cast<T*>(slab + frag_row * SLAB_STRIDE) + 8 * q + 4 * half_sel);
 						}
 						wait_lgkmcnt_zero(); /* the slab is private to this wavefront */
@@ -317,8 +369,8 @@ namespace mlhip
 							const int row = pass * ROWS_PER_PASS + lane / LANES_PER_ROW;
 							const uint4_t v = *reinterpret_cast<const uint4_t*>(slab + row * SLAB_STRIDE + col * sizeof(T));
 							const int m = m_first + 32 * i + row;
-							if (m < M && n0 + col < N) /* N is a multiple of the 16-byte vector (checked by the launcher) */
-								*reinterpret_cast<uint4_t*>(c_base + static_cast<size_t>(m) * N + n0 + col) = v;
+							if (m < M && n0 + col < out_n) /* the width is a multiple of the 16-byte vector (checked by the launcher) */
+								*reinterpret_cast<uint4_t*>(out_base + static_cast<size_t>(m) * out_stride + n0 + col) = v;
 						}
 						wait_lgkmcnt_zero();
 						__builtin_amdgcn_wave_barrier();
@@ -434,6 +486,7 @@ namespace mlhip
 			void *C; /* used by PlainStore only; functors carry their own pointers */
 			int M, N, k_bytes, batch;
 			size_t stride_a, stride_b, stride_c;
+			size_t a_row_bytes = 0; /* bytes between consecutive rows of A; 0 = dense rows of k_bytes */
 	};
 	/*
 	 * A K row length the kernel is instantiated for. There is no lower bound on the size of the product: with a single unit per
@@ -459,7 +512,7 @@ namespace mlhip
 		typedef StreamGemmConfig Cfg;
 		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
 		constexpr int WAVES = WAVES_M * WAVES_N;
-		constexpr int SLAB_BYTES = WAVES * 32 * (32 * (PLAIN ? sizeof(T) : 4) + 16);
+		constexpr int SLAB_BYTES = WAVES * 32 * (32 * (stream_epilogue_reads_nothing<Epilogue>::value ? sizeof(T) : 4) + 16);
 		constexpr int STAGES = (8 * Cfg::STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? 8 : 7;
 		constexpr int LDS = STAGES * Cfg::STAGE_BYTES + SLAB_BYTES;
 		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
@@ -491,14 +544,17 @@ namespace mlhip
 			}
 		}
 		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
-				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, sweep, epilogue);
+				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, sweep,
+				g.a_row_bytes != 0 ? g.a_row_bytes : static_cast<size_t>(KB), epilogue);
 	}
 	/* wavefront layout by output width: 8 x 32 columns for N > 128, 2 x 4 for N > 64, 4 x 2 below */
 	template<typename T, int KB, typename Epilogue>
 	inline void launch_stream_gemm_kb(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
 	{
 		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
-		constexpr bool WIDE_FITS = PLAIN || KB < 512; /* else B-operand registers + side inputs + a 128-row accumulator exceed 256 VGPRs */
+		/* else B-operand registers + side inputs + a 128-row accumulator exceed 256 VGPRs (at 512 bytes an epilogue that reads nothing per
+		 * element still fits: 233) */
+		constexpr bool WIDE_FITS = PLAIN || KB < 512 || (KB == 512 && stream_epilogue_reads_nothing<Epilogue>::value);
 		/* slices of 256 columns unless slices of 128 pad N less (N = 384: two wide slices multiply 512 columns, three narrow ones 384;
 		 * measured 252 -> 206 us for the Winograd product at 384 channels) */
 		const bool wide_pads_more = ceil_div(g.N, 256) * 256 > ceil_div(g.N, 128) * 128;
@@ -517,6 +573,16 @@ namespace mlhip
 	template<typename T, typename Epilogue>
 	inline void launch_stream_gemm(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
 	{
+		if constexpr (!std::is_same<Epilogue, PlainStore>::value && stream_epilogue_reads_nothing<Epilogue>::value)
+		{
+			/* the packed form stores 16 bytes per lane: rows and widths that do not allow it take the functor's run-time form */
+			const auto sixteen = [](size_t elements) { return (elements * sizeof(T)) % 16 == 0; };
+			if (!(sixteen(epilogue.N) && sixteen(epilogue.row_stride) && sixteen(g.stride_c) && reinterpret_cast<uintptr_t>(epilogue.D) % 16 == 0))
+			{
+				launch_stream_gemm<T>(stream, g, epilogue.template fixed<EPILOGUE_RUNTIME, EPILOGUE_RUNTIME, EPILOGUE_RUNTIME>());
+				return;
+			}
+		}
 		switch (g.k_bytes)
 		{
 			case 128:

@@ -17,6 +17,7 @@
 #include "device_utils.hpp"
 #include "epilogues.hpp"
 #include "gemm_dma.hpp"
+#include "gemm_stream.hpp"
 
 namespace
 {
@@ -661,8 +662,18 @@ extern "C"
 				if constexpr (sizeof(T) == 2)
 					specialise_epilogue(ep, [&](const auto &fixed)
 					{
-						launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
-								static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), fixed);
+						if (vectorized && stream_gemm_half_applies(static_cast<int>(rows), experts, k_bytes))
+						{
+							/* short K rows (the layer that widens 256 channels to the hidden width): the streaming kernel, whose B operand
+							 * stays in registers; the experts are the matrices of its batch, their rows E * C elements apart */
+							StreamGemmArgs sg { x.data, w.data, y.data, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts,
+									static_cast<size_t>(channels), static_cast<size_t>(neurons) * channels, static_cast<size_t>(neurons) };
+							sg.a_row_bytes = static_cast<size_t>(experts) * k_bytes;
+							launch_stream_gemm<T>(stream, sg, fixed);
+						}
+						else
+							launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
+									static_cast<size_t>(neurons) * k_bytes, static_cast<size_t>(neurons), fixed);
 					});
 				else
 					launch_gemm_dma<T>(stream, a_loader, b_loader, static_cast<int>(rows), neurons, static_cast<int>(k_bytes), experts, k_bytes,
