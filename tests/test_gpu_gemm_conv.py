@@ -159,6 +159,15 @@ def test_gemm_ex_streaming_shapes(ctx, dtype, k_bytes, M, N):
     dD = ml.toDevice(ctx, C)
     ml.gemm_ex(ctx, dD, 1.0, "n", dA, "t", dB, 1.0, dD, None, "sigmoid")
     assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, alpha=1.0, beta=1.0, C=C, act=O.SIGMOID)) <= TOL[dtype]
+    # epilogues that read nothing per element (no C): in fp16 they are finished in registers and stored 16 bytes per lane when the
+    # width allows it (N = 100 and 28 do not: the functor's run-time form)
+    dbias = ml.toDevice(ctx, bias)
+    for alpha, use_bias, act in ((0.9, True, "relu"), (1.0, True, "linear"), (0.9, False, "linear")):
+        dD = ml.Tensor((M, N), dtype)
+        dD.setall(ctx, float("nan"))
+        ml.gemm_ex(ctx, dD, alpha, "n", dA, "t", dB, 0.0, None, dbias if use_bias else None, act)
+        want = O.gemm(A, Bm, alpha=alpha, bias=bias if use_bias else None, act=ml.act_of(act))
+        assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
