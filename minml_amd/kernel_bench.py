@@ -449,12 +449,47 @@ def library(reps):
 
 
 
+def streams(steps=10):
+    """The 20 x 256 fp16 network on several contexts (HIP streams) of the one device, every stream with its own network object and
+    workspace: a batch of 1024 positions split into 2 or 4 equal parts, or two whole batches of 1024 in flight at once. While one stream's
+    launch starts up or drains, another's is in its steady state. Prints wall-clock positions per second (repeated rows show drift)."""
+    import time
+    from .resnet import ResNet, make_input, make_parameters
+    to_storage = lambda a: np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
+    params = make_parameters(1, 32, 256, 20)
+    x = to_storage(make_input(1, 1024, 15, 32))
+    for parts, per in ((1, 1024), (2, 512), (4, 256), (2, 1024), (2, 512), (1, 1024), (2, 1024)):
+        contexts = [ml.Context(0) for _ in range(parts)]
+        nets = [ResNet(c, per, 15, 32, 256, 20, "float16", params, to_storage, fused=True) for c in contexts]
+        for i, net in enumerate(nets):
+            net.setInput(x[(i * per) % 1024:(i * per) % 1024 + per])
+        def one_pass():
+            for net in nets:
+                net.forward()
+        for _ in range(3):
+            one_pass()
+        for c in contexts:
+            c.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one_pass()
+        for c in contexts:
+            c.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        print("streams   cfg2 network, %d x %4d positions on %d stream(s): %7.3f ms per round of passes, %7.0f positions/s"
+              % (parts, per, parts, dt * 1e3, parts * per / dt), flush=True)
+        del nets, contexts
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library", "streams"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
+    if args.group == "streams":  # only on request: whole passes on several streams, wall-clock
+        streams()
+        return 0
     if args.group == "library":  # only on request: a yardstick that needs PyTorch
         print("%-9s %-34s %-34s %12s  %-4s %9s %-7s  %7s" % ("group", "entry point", "shape", "time", "bnd", "achieved", "", "of peak"))
         library(args.reps)
