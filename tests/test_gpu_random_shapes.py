@@ -271,3 +271,123 @@ def test_mixture_of_experts_random(ctx, seed):
     dy = ml.toDevice(ctx, y0)
     ml.scatterTokensForward(ctx, ml.toDevice(ctx, want_hidden), d_iv, 1.0, dy)
     assert max_abs_rel(dy.copyToHost(ctx), M.scatter_tokens(want_hidden, want_iv, (b, h, w, n), beta=1.0, y=y0)) <= TOL[dtype], case
+
+
+# ---- the same entry points on tensors that do not start at an aligned address --------------------------------------------------------
+# The reference hands the backend views into larger allocations (Tensor::view: the layer workspace is cut into the three Winograd
+# matrices at element offsets, src/layers/Conv2D.cpp:365-367), so a pointer may be aligned to its element size only. The vector forms of
+# every kernel check the addresses they are given; these cases give each operand its own small element offset.
+
+def _np_dtype_name(array):
+    return {np.dtype(np.uint16): "float16", np.dtype(np.float32): "float32", np.dtype(np.int8): "int8", np.dtype(np.int32): "int32"}[array.dtype]
+
+
+def _at(ctx, array, offset):
+    """device copy of `array` that starts `offset` elements into its allocation"""
+    base = ml.Tensor((array.size + offset,), _np_dtype_name(array))
+    view = base.view(array.shape, offset)
+    view.copyFromHost(ctx, array)
+    return view
+
+
+def _out_at(ctx, shape, dtype, offset):
+    base = ml.Tensor((int(np.prod(shape)) + offset,), dtype)
+    view = base.view(shape, offset)
+    if dtype in ("float32", "float16"):
+        view.setall(ctx, float("nan"))
+    return view
+
+
+def _offsets(rng, count):
+    return [int(rng.choice([0, 1, 2, 3, 4, 5, 8])) for _ in range(count)]
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_gemm_ex_on_offset_views(ctx, seed):
+    rng = np.random.default_rng(9000 + seed)
+    dtype = ["float32", "float16"][seed % 2]
+    esize = 4 if dtype == "float32" else 2
+    K = max(1, int(rng.choice(K_BYTES)) // esize)
+    M, N = _draw_extent(rng, 500), _draw_extent(rng, 280)
+    beta = float(rng.choice([0.0, 0.5]))
+    use_bias = bool(rng.integers(0, 2))
+    act = ["linear", "relu"][int(rng.integers(0, 2))]
+    oa, ob, oc, od, obias = _offsets(rng, 5)
+    case = "seed %d: %s M=%d N=%d K=%d beta=%g bias=%s act=%s offsets A %d B %d C %d D %d bias %d" % (seed, dtype, M, N, K, beta, use_bias, act, oa, ob, oc,
+                                                                                                 od, obias)
+    A = random_tensor(rng, (M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (N, K), dtype, (1.0 / K) ** 0.5)
+    C = random_tensor(rng, (M, N), dtype)
+    bias = random_tensor(rng, (N,), dtype)
+    dD = _out_at(ctx, (M, N), dtype, od)
+    ml.gemm_ex(ctx, dD, 1.0, "n", _at(ctx, A, oa), "t", _at(ctx, Bm, ob), beta, _at(ctx, C, oc) if beta != 0.0 else None,
+               _at(ctx, bias, obias) if use_bias else None, act)
+    want = O.gemm(A, Bm, alpha=1.0, beta=beta, C=C if beta != 0.0 else None, bias=bias if use_bias else None, act=ml.act_of(act))
+    assert max_abs_rel(dD.copyToHost(ctx), want) <= TOL[dtype], case
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_gemm_batched_on_offset_views(ctx, seed):
+    rng = np.random.default_rng(9500 + seed)
+    dtype = ["float32", "float16"][seed % 2]
+    esize = 4 if dtype == "float32" else 2
+    K = max(1, int(rng.choice(K_BYTES)) // esize)
+    batch = int(rng.choice([1, 3, 36]))
+    M, N = _draw_extent(rng, 300), _draw_extent(rng, 260)
+    oa, ob, oc = _offsets(rng, 3)
+    case = "seed %d: %s batch=%d M=%d N=%d K=%d offsets A %d B %d C %d" % (seed, dtype, batch, M, N, K, oa, ob, oc)
+    A = random_tensor(rng, (batch, M, K), dtype, 0.5)
+    Bm = random_tensor(rng, (batch, N, K), dtype, (1.0 / K) ** 0.5)
+    dC = _out_at(ctx, (batch, M, N), dtype, oc)
+    ml.gemmBatched(ctx, "n", "t", dC, _at(ctx, A, oa), _at(ctx, Bm, ob), 1.0, 0.0)
+    got = dC.copyToHost(ctx)
+    for i in range(batch):
+        assert max_abs_rel(got[i], O.gemm(A[i], Bm[i])) <= TOL[dtype], case + " matrix %d" % i
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_convolutions_on_offset_views(ctx, seed):
+    """the float convolution, the int8 convolution and the Winograd transforms with every operand at its own offset"""
+    rng = np.random.default_rng(9800 + seed)
+    dtype = ["float32", "float16"][seed % 2]
+    k = int(rng.choice([1, 3, 5]))
+    b, h, w = int(rng.integers(1, 3)), int(rng.integers(1, 17)), int(rng.integers(1, 17))
+    cin = int(rng.choice([3, 8, 16, 32, 64, 128, 256]))
+    cout = _draw_extent(rng, 130)
+    ox, ow, ob, oe, oy = _offsets(rng, 5)
+    case = "seed %d: %s [%d,%d,%d,%d] -> %d k=%d offsets x %d w %d bias %d ext %d y %d" % (seed, dtype, b, h, w, cin, cout, k, ox, ow, ob, oe, oy)
+    x = random_tensor(rng, (b, h, w, cin), dtype)
+    wt = random_tensor(rng, (cout, k, k, cin), dtype, (2.0 / (k * k * cin)) ** 0.5)
+    bias = random_tensor(rng, (cout,), dtype)
+    add = random_tensor(rng, (b, h, w, cout), dtype)
+    dy = _out_at(ctx, (b, h, w, cout), dtype, oy)
+    ml.convolutionImplicitGemmForward(ctx, _at(ctx, x, ox), _at(ctx, wt, ow), dy, _at(ctx, bias, ob), _at(ctx, add, oe), "relu")
+    assert max_abs_rel(dy.copyToHost(ctx), O.conv2d_forward(x, wt, bias, add, O.RELU)) <= TOL[dtype], case
+    # int8, bit for bit
+    xq = rng.integers(-128, 128, (b, h, w, cin)).astype(np.int8)
+    wq = rng.integers(-127, 128, (cout, k, k, cin)).astype(np.int8)
+    scales = (rng.random(cout) * 0.002 + 0.0005).astype(np.float32)
+    fbias = rng.standard_normal(cout).astype(np.float32)
+    ext = rng.integers(-128, 128, (b, h, w, cout)).astype(np.int8)
+    in_qd, out_qd, ext_qd = (0.123, 4.56), (0.078, 0.9), (0.078, -0.9)
+    dq = _out_at(ctx, (b, h, w, cout), "int8", oy)
+    ml.quantizedConvForward(ctx, _at(ctx, xq, ox), in_qd, _at(ctx, wq, ow), _at(ctx, scales, ob), _at(ctx, fbias, oe), dq, out_qd, _at(ctx, ext, oe),
+                            ext_qd, "relu")
+    want = O.int8_conv2d_forward(xq, in_qd, wq, scales, fbias, O.INT8, out_qd, ext, ext_qd, O.RELU)
+    assert mismatches(dq.copyToHost(ctx), want) == 0, case
+    # Winograd transforms of the same tensors, bit for bit
+    tiles = b * ((h + 3) // 4) * ((w + 3) // 4)
+    dv = _out_at(ctx, (36, tiles, cin), dtype, oy)
+    ml.winogradInputTransform(ctx, (cout, 3, 3, cin), _at(ctx, x, ox), dv)
+    assert mismatches(dv.copyToHost(ctx), O.winograd_input_transform(x)) == 0, case
+    m = random_tensor(rng, (36, tiles, cout), dtype)
+    want_y = O.winograd_output_transform(m, (b, h, w, cout), bias, add, O.RELU)
+    dy = _out_at(ctx, (b, h, w, cout), dtype, oy)
+    dm = _at(ctx, m, ow)
+    ml.winogradOutputTransform(ctx, (cout, 3, 3, cout), dm, dy, _at(ctx, bias, ob), _at(ctx, add, oe), O.RELU)
+    assert mismatches(dy.copyToHost(ctx), want_y) == 0, case
+    dy2 = _out_at(ctx, (b, h, w, cout), dtype, oy)
+    dv2 = _out_at(ctx, (36, tiles, cout), dtype, ox)
+    ml.winogradOutputInputTransform(ctx, (cout, 3, 3, cout), dm, (b, h, w, cout), dy2, _at(ctx, bias, ob), _at(ctx, add, oe), O.RELU, dv2)
+    assert mismatches(dy2.copyToHost(ctx), want_y) == 0, case
+    assert mismatches(dv2.copyToHost(ctx), O.winograd_input_transform(want_y)) == 0, case
