@@ -123,8 +123,10 @@ namespace mlhip
 	 * One workgroup of WAVES_M x WAVES_N wavefronts covers a unit of 128 rows x 32 * WAVES_N columns; a wavefront owns 128 / WAVES_M
 	 * rows x 32 columns, keeps the B operand of its 32 columns (KB bytes of K each) in KB / 8 VGPRs and accumulates in 32x32 blocks; the
 	 * pipeline is one k step deep. KB = 128, 256 or 512 bytes per K row. Epilogue: PlainStore, or a functor with the split protocol of
-	 * epilogues.hpp (load_column / load_extra / apply on 4 consecutive n, vectorized case only), whose D / C pointers advance by
-	 * stride_c per matrix of the batch.
+	 * epilogues.hpp (load_column / load_extra / apply on 4 consecutive n, vectorized case only; value() instead of apply() for functors
+	 * that read nothing per element), whose D / C pointers advance by stride_c and whose bias advances by its bias_batch_stride per
+	 * matrix of the batch. Consecutive rows of A lie a_row_bytes apart (KB for a dense matrix; more when the matrices of the batch are
+	 * interleaved row by row, as the experts' tokens are).
 	 */
 	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue>
 	__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a,
