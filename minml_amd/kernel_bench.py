@@ -481,12 +481,47 @@ def streams(steps=10):
         del nets, contexts
 
 
+def latency(reps=50):
+    """The 20 x 256 fp16 network at small batches (1 ... 512 positions per pass): wall-clock time of a pass issued call by call from
+    this Python mirror, and of the same pass recorded once and replayed as one HIP graph (hip_graph_*). Below about 128 positions a
+    pass is a chain of dependent launches of a few microseconds each; the replay removes the host's share of it."""
+    import time
+    from .resnet import ResNet, make_input, make_parameters
+    to_storage = lambda a: np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
+    params = make_parameters(1, 32, 256, 20)
+    ctx = ml.Context(0)
+    for batch in (1, 8, 32, 64, 128, 256, 512):
+        net = ResNet(ctx, batch, 15, 32, 256, 20, "float16", params, to_storage, fused=True)
+        net.setInput(to_storage(make_input(1, batch, 15, 32)))
+        n = reps if batch <= 128 else max(1, reps // 5)
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            ctx.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            ctx.synchronize()
+            return (time.perf_counter() - t0) / n
+        eager = timed(net.forward)
+        graph = ml.Graph.record(ctx, net.forward)
+        replayed = timed(graph.launch)
+        graph.destroy()
+        print("latency   cfg2 network, %4d positions per pass: call by call %7.3f ms, recorded and replayed %7.3f ms (%7.0f -> %7.0f positions/s)"
+              % (batch, eager * 1e3, replayed * 1e3, batch / eager, batch / replayed), flush=True)
+        del net
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library", "streams"])
+    ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library", "streams", "latency"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
+    if args.group == "latency":  # only on request: whole passes at small batches, wall-clock
+        latency()
+        return 0
     if args.group == "streams":  # only on request: whole passes on several streams, wall-clock
         streams()
         return 0
