@@ -349,6 +349,17 @@ class Bench:
                 report("read stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, None, a.ptr, nbytes, 0, nt, wgs)), nbytes)
                 report("write stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, None, nbytes, 1, nt, wgs)), nbytes)
                 report("copy stream (read + write)" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, a.ptr, nbytes, 2, nt, wgs)), 2 * nbytes)
+            if size_mib == 1024:
+                # the same streams cut into 16 KiB pieces, one per workgroup, handed out in address order: at any moment the resident
+                # workgroups cover one dense window of memory instead of 2048 separate positions
+                fine = nbytes // (16 * 1024)
+                for nt in (0, 1):
+                    tag = " (non-temporal)" if nt else ""
+                    shape = "%d MiB, HBM, 16 KiB per workgroup" % size_mib
+                    report("read stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, None, a.ptr, nbytes, 0, nt, fine)), nbytes)
+                    report("write stream" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, None, nbytes, 1, nt, fine)), nbytes)
+                    report("copy stream (read + write)" + tag, shape, self.time(lambda: lib.ceil_stream(stream, b.ptr, a.ptr, nbytes, 2, nt, fine)),
+                           2 * nbytes)
             a.free()
             b.free()
         # producer -> consumer chains: launch i reads what launch i-1 wrote; three buffers in rotation
@@ -446,6 +457,29 @@ def library(reps):
     row("torch.matmul (square)", 8192, 8192, 8192, "float16")
     row("torch._int_mm (cfg3 3x3 C=256 as GEMM)", 230400, 256, 2304, "int8")
     row("torch._int_mm (square)", 8192, 8192, 8192, "int8")
+
+    # the same for memory streams: PyTorch's own copy and element-wise kernels on tensors beyond the last-level cache
+    def stream_row(name, fn, nbytes):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(reps):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        t = start.elapsed_time(end) / reps * 1e-3
+        print("%-9s %-34s %-34s %9.1f us  %-4s %9.1f %-7s  %5.1f %%" % ("library", name, "%d MiB moved per call" % (nbytes >> 20), t * 1e6, "hbm",
+                                                                        nbytes / t / 1e9, "GB/s", 100 * nbytes / t / PEAK["hbm"]), flush=True)
+    n = 1 << 29  # halfs: 1 GiB per tensor
+    x = torch.randn(n, dtype=torch.float16, device=dev)
+    y = torch.empty_like(x)
+    z = torch.randn(n, dtype=torch.float16, device=dev)
+    stream_row("torch copy_ (1 GiB -> 1 GiB)", lambda: y.copy_(x), 2 * n * 2)
+    stream_row("torch add (2 x 1 GiB -> 1 GiB)", lambda: torch.add(x, z, out=y), 3 * n * 2)
+    stream_row("torch relu_ in place (1 GiB)", lambda: torch.relu_(y), 2 * n * 2)
+    stream_row("torch sum (1 GiB read)", lambda: x.sum(), n * 2)
+    stream_row("torch fill_ (1 GiB written)", lambda: y.fill_(1.0), n * 2)
 
 
 
