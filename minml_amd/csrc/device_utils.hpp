@@ -229,6 +229,20 @@ namespace mlhip
 			return id; /* tail blocks keep their id */
 		return (id % XCDS) * (full / XCDS) + id / XCDS;
 	}
+	/*
+	 * The other way to keep neighbouring work in one L2: runs of `run` consecutive logical ids go to one XCD, and the runs go round
+	 * the 8 XCDs, so that the whole chip works on one dense window of the logical range at any moment. Ids beyond the last whole
+	 * group of 8 runs keep their value.
+	 */
+	__device__ __forceinline__ unsigned int xcd_run_block_id(unsigned int id, unsigned int count, unsigned int run)
+	{
+		constexpr unsigned int XCDS = 8;
+		const unsigned int span = XCDS * run, full = count / span * span;
+		if (id >= full)
+			return id;
+		const unsigned int xcd = id % XCDS, seq = id / XCDS;
+		return (seq / run) * span + xcd * run + seq % run;
+	}
 } /* namespace mlhip */
 
 #endif /* MINML_AMD_DEVICE_UTILS_HPP_ */
