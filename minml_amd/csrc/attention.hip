@@ -261,8 +261,11 @@ namespace
 		uint32_t *place = reinterpret_cast<uint32_t*>(lds + Lds::place_offset(tokens));
 		float *bias = reinterpret_cast<float*>(lds + Lds::table_offset(tokens));
 
-		const int image = blockIdx.x / shape.heads;
-		const int head = blockIdx.x - image * shape.heads;
+		/* the heads of one image run on one XCD (images go round the XCDs): their q / k / v parts are neighbouring pieces of the same
+		 * token rows, which then meet in one L2 instead of being fetched through eight */
+		const unsigned int lin = (shape.heads > 1) ? xcd_run_block_id(blockIdx.x, gridDim.x, shape.heads) : blockIdx.x;
+		const int image = lin / shape.heads;
+		const int head = lin - image * shape.heads;
 		const T *tokens_base = input + static_cast<size_t>(image) * tokens * shape.token_stride + head * D;
 		const int range = (shape.table_size - 1) / 2;
 		/* scores are kept in units of ln 2 (scale and table carry the factor log2 e) so that the exponential is the hardware's exp2 */
