@@ -2,9 +2,10 @@
  * ceilings.hip — probes of what one MI355X sustains, independent of the backend's kernels: plain read / write / copy streams over a
  * buffer of a given size (HBM when the buffer exceeds the 256 MB last-level cache, that cache or the L2s when it fits) and a pure MFMA
  * loop on operands held in registers. Built as its own small library (libminml_ceilings.so) and used only by
- * `python3 -m minml_amd.kernel_bench --group ceilings`; nothing in the backend library depends on it.
+ * `python3 kernel_bench.py --group ceilings` (which also builds it: --build-ceilings); nothing in the backend library depends on it.
  *
- * The entry points take a hipStream_t and raw device pointers and launch one kernel each; the caller times them with events.
+ * The entry points take a hipStream_t and raw device pointers and launch one kernel each; the caller times them with events. They are
+ * called through ctypes, so no exception may leave them: each returns 0, or -1 after storing a message that ceil_last_error() returns.
  */
 #include <hip/hip_runtime.h>
 
@@ -207,10 +208,33 @@ namespace
 	}
 }
 
+namespace
+{
+	std::string last_error;
+	template<typename F>
+	int guarded(F &&body)
+	{
+		try
+		{
+			body();
+			return 0;
+		}
+		catch (const std::exception &e)
+		{
+			last_error = e.what();
+		}
+		catch (...)
+		{
+			last_error = "ceilings: unknown failure";
+		}
+		return -1;
+	}
+}
+
 extern "C"
 {
 	/* v: 36 * tiles * 512 bytes, u: 36 * columns * 512 bytes; tile_group x column_slice is 32 x 64 or 64 x 32; returns the bytes one launch moves */
-	size_t ceil_fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups)
+	static size_t fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups)
 	{
 		if (tiles <= 0 || columns <= 0 || tiles % tile_group != 0 || columns % column_slice != 0 || workgroups <= 0)
 			throw std::logic_error("ceilings: ceil_fused_layer_operand_stream: bad arguments");
@@ -237,7 +261,7 @@ extern "C"
 	}
 
 	/* mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16; nt != 0 uses non-temporal accesses */
-	void ceil_stream(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
+	static void stream_launch(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
 	{
 		if (bytes % 16 != 0 || workgroups <= 0 || mode < 0 || mode > 2)
 			throw std::logic_error("ceilings: ceil_stream: bad arguments");
@@ -262,7 +286,7 @@ extern "C"
 		check(hipGetLastError(), "launch of kernel_stream");
 	}
 	/* one launch of the MFMA loop on `workgroups` workgroups of 4 wavefronts; `out` = at least 2 + 256 uint64 of device memory */
-	void ceil_mfma(void *stream, void *out, int iters, int random, int int8 /* 0 fp16, 1 int8, 2 fp32 */, int workgroups)
+	static void mfma_launch(void *stream, void *out, int iters, int random, int int8 /* 0 fp16, 1 int8, 2 fp32 */, int workgroups)
 	{
 		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 		if (int8 == 1)
@@ -272,5 +296,24 @@ extern "C"
 		else
 			hipLaunchKernelGGL(kernel_mfma_loop<0>, dim3(workgroups), dim3(256), 0, s, reinterpret_cast<uint64_t*>(out), iters, random);
 		check(hipGetLastError(), "launch of kernel_mfma_loop");
+	}
+
+	const char* ceil_last_error()
+	{
+		return last_error.c_str();
+	}
+	/* *bytes_moved receives the bytes one launch brings into LDS */
+	int ceil_fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups,
+			size_t *bytes_moved)
+	{
+		return guarded([&]() { *bytes_moved = fused_layer_operand_stream(stream, v, u, tiles, columns, tile_group, column_slice, workgroups); });
+	}
+	int ceil_stream(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
+	{
+		return guarded([&]() { stream_launch(stream, dst, src, bytes, mode, nt, workgroups); });
+	}
+	int ceil_mfma(void *stream, void *out, int iters, int random, int int8, int workgroups)
+	{
+		return guarded([&]() { mfma_launch(stream, out, iters, random, int8, workgroups); });
 	}
 }

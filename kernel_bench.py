@@ -1,4 +1,4 @@
-"""Per-kernel roofline table of the convolution / GEMM path on one MI355X:  python3 -m minml_amd.kernel_bench [--group NAME] [--json]
+"""Per-kernel roofline table of the convolution / GEMM path on one MI355X:  python3 kernel_bench.py [--group NAME] [--json]
 
 Every row launches one entry point of the library on synthetic tensors of a benchmark configuration's shape (resident in HBM), times
 `--reps` launches with two events on the context's stream, and prices the launch with its ALGORITHMIC work: the bytes every
@@ -12,7 +12,8 @@ misc (im2row, element-wise neighbours), heads (softmax, global average pooling, 
 (RMS normalisation and multi-head attention at the hybrid configuration's shape), moe (routing, gather, the two expert layers and
 scatter of that configuration's mixture-of-experts half-block), ceilings (what the chip sustains independent of the
 backend's kernels: read / write / copy streams over buffers that fit the L2s, the 256 MB last-level cache or neither, and a pure MFMA
-loop on constant and on random operands with the shader clock it ran at; needs libminml_ceilings.so, built by minml_amd.build),
+loop on constant and on random operands with the shader clock it ran at; its probe kernels are ceilings.hip beside this file, compiled into libminml_ceilings.so by
+`python3 kernel_bench.py --build-ceilings`, which __graft_entry__.build() also runs),
 library (only on request, needs PyTorch: the vendor GEMM library on plain dense products of the convolutions' shapes, as a yardstick).
 """
 import argparse
@@ -23,7 +24,9 @@ import sys
 
 import numpy as np
 
-from . import core as ml
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+from minml_amd import core as ml  # noqa: E402
 
 PEAK = {"hbm": 8000.0e9, "float16": 2500.0e12, "float32": 157.3e12, "int8": 5000.0e12}
 ESIZE = {"float16": 2, "float32": 4, "int8": 1, "int32": 4}
@@ -316,15 +319,31 @@ class Bench:
         ctx = self.ctx
         path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libminml_ceilings.so")
         if not os.path.exists(path):
-            raise RuntimeError("%s is missing: build it with `python -m minml_amd.build`" % path)
-        lib = ctypes.CDLL(path)
+            raise RuntimeError("%s is missing: build it with `python3 kernel_bench.py --build-ceilings`" % path)
+        raw = ctypes.CDLL(path)
         vp = ctypes.c_void_p
-        lib.ceil_stream.argtypes = [vp, vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        lib.ceil_stream.restype = None
-        lib.ceil_mfma.argtypes = [vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        lib.ceil_mfma.restype = None
-        lib.ceil_fused_layer_operand_stream.argtypes = [vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        lib.ceil_fused_layer_operand_stream.restype = ctypes.c_size_t
+        raw.ceil_last_error.restype = ctypes.c_char_p
+
+        class Checked:
+            """The probe library's entry points return 0 or -1 (message from ceil_last_error): a failure raises here."""
+
+            def __init__(self, **argtypes):
+                for name, types in argtypes.items():
+                    fn = getattr(raw, name)
+                    fn.argtypes, fn.restype = types, ctypes.c_int
+                    setattr(self, name, self._wrap(name, fn))
+
+            @staticmethod
+            def _wrap(name, fn):
+                def call(*args):
+                    if fn(*args) != 0:
+                        raise RuntimeError("%s: %s" % (name, raw.ceil_last_error().decode()))
+                return call
+
+        lib = Checked(ceil_stream=[vp, vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int],
+                      ceil_mfma=[vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int],
+                      ceil_fused_layer_operand_stream=[vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                                       ctypes.POINTER(ctypes.c_size_t)])
         stream = ctx.stream()
         mib = 1 << 20
 
@@ -385,9 +404,9 @@ class Bench:
         v.zeroall(ctx)
         u.zeroall(ctx)
         for group, width in ((32, 64), (64, 32)):
-            moved = []
-            t = self.time(lambda: moved.append(lib.ceil_fused_layer_operand_stream(stream, v.ptr, u.ptr, tiles, columns, group, width, 256)))
-            report("one-kernel Winograd layer: operands", "%d tiles x %d columns x 36 per task" % (group, width), t, moved[-1])
+            moved = ctypes.c_size_t(0)
+            t = self.time(lambda: lib.ceil_fused_layer_operand_stream(stream, v.ptr, u.ptr, tiles, columns, group, width, 256, ctypes.byref(moved)))
+            report("one-kernel Winograd layer: operands", "%d tiles x %d columns x 36 per task" % (group, width), t, moved.value)
         v.free()
         u.free()
         out8 = ml.Tensor((4096,), "uint8")
@@ -488,7 +507,7 @@ def streams(steps=10):
     workspace: a batch of 1024 positions split into 2 or 4 equal parts, or two whole batches of 1024 in flight at once. While one stream's
     launch starts up or drains, another's is in its steady state. Prints wall-clock positions per second (repeated rows show drift)."""
     import time
-    from .resnet import ResNet, make_input, make_parameters
+    from minml_amd.resnet import ResNet, make_input, make_parameters
     to_storage = lambda a: np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
     params = make_parameters(1, 32, 256, 20)
     x = to_storage(make_input(1, 1024, 15, 32))
@@ -520,7 +539,7 @@ def latency(reps=50):
     this Python mirror, and of the same pass recorded once and replayed as one HIP graph (hip_graph_*). Below about 128 positions a
     pass is a chain of dependent launches of a few microseconds each; the replay removes the host's share of it."""
     import time
-    from .resnet import ResNet, make_input, make_parameters
+    from minml_amd.resnet import ResNet, make_input, make_parameters
     to_storage = lambda a: np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
     params = make_parameters(1, 32, 256, 20)
     ctx = ml.Context(0)
@@ -547,12 +566,32 @@ def latency(reps=50):
         del net
 
 
+def build_ceilings(verbose=False):
+    """Compiles ceilings.hip (beside this file) into libminml_ceilings.so (beside this file) for gfx950, with the backend's flags."""
+    import subprocess
+    from minml_amd.build import COMMON, hipcc
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    out = os.path.join(here, "libminml_ceilings.so")
+    cmd = [hipcc()] + COMMON + ["-shared", os.path.join(here, "ceilings.hip"), "-o", out]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), res.stdout))
+    if verbose:
+        print("built", out)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--build-ceilings", action="store_true", help="compile the probe kernels of the ceilings group and exit")
     ap.add_argument("--group", default="all", choices=["all", "winograd", "small", "conv", "int8", "misc", "heads", "transformer", "moe", "ceilings", "library", "streams", "latency"])
     ap.add_argument("--reps", type=int, default=10)
     ap.add_argument("--json", action="store_true", help="print one JSON object per row after the table")
     args = ap.parse_args()
+    if args.build_ceilings:
+        build_ceilings(verbose=True)
+        return 0
     if args.group == "latency":  # only on request: whole passes at small batches, wall-clock
         latency()
         return 0

@@ -12,9 +12,6 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libminml_hip.so")
-# hardware-ceiling probes for the per-kernel benchmark (read / write / copy streams, a pure MFMA loop): a library of its own, so that
-# the backend library exports nothing but the backend's interface
-CEILINGS_LIB = os.path.join(HERE, "libminml_ceilings.so")
 
 SOURCES = ["runtime.hip", "winograd.hip", "gemm.hip", "conv.hip", "quantized.hip", "elementwise.hip", "heads.hip", "attention.hip", "moe.hip", "cuda_stubs.cpp"]
 # packed fp32 VALU forms are switched off for all device code; the host pass does not know the feature and says so (harmless)
@@ -55,9 +52,8 @@ def build(verbose=False, jobs=None):
         return obj
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(compile_one, SOURCES + ["ceilings.hip"]))
-    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs[:-1])
-    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", CEILINGS_LIB, objs[-1]])
+        objs = list(pool.map(compile_one, SOURCES))
+    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
     return LIB
 
 
