@@ -20,6 +20,16 @@ layer). Prints ONE JSON line:
                its sources (kind "reference", one thread, as the reference runs) when that library is present, otherwise this
                repository's C restatement (kind "port")
 
+  reference_call_sequence   the same batch through the reference's own call sequence (three calls per 3x3 layer: input transform, batched GEMM,
+               output transform; src/layers/Conv2D.cpp:365-378) — what the timed `value` gains over it is the cross-layer transform fusion,
+               an entry point that no unchanged minml caller uses
+  dropin_graph_predict      the reference's own Graph / Conv2D / dispatcher code (compiled from its sources into oracle/_ref/dropin_graph and linked
+               against this backend in place of its CUDA backend) timed the way its launcher times a network (launcher/minml.cpp:3924-3936:
+               predict + synchronize in a loop): the throughput an unchanged minml gets. Run as a child process before this process touches the GPU.
+
+--config cfg4_conv_sweep_fp16_b512 runs the implicit-GEMM convolution sweep (19x19 boards, batch 512, 64 / 128 / 256 / 384 channels, kernels
+1 / 3 / 5, bias + residual + ReLU fused): a step is the 12 layers one after the other; `rows` prices each against its own roofline.
+
 --config cfg3_resnet20x256_int8_b1024 runs the int8 form of the same network instead (per-channel int8 weights, per-tensor int8
 activations calibrated on 64 random batches, every 3x3 layer one fused int8 implicit-GEMM convolution with int32 accumulation and
 requantisation); its roofline object prices that convolution against the dense int8 MFMA peak (5 POP/s).
@@ -50,6 +60,41 @@ CONFIGS = {
     "cfg5_hybrid10x256_attention4_moe8_fp16_b256": (256, 15, 32, 256, 10, "hybrid_moe", 4),
 }
 PEAK_INT8_TOPS = 5000.0
+CONV_SWEEP = "cfg4_conv_sweep_fp16_b512"
+
+
+def run_dropin_graph(batch, channels, blocks, dtype, seconds):
+    """Spawns oracle/_ref/dropin_graph (the reference's Graph on this backend) in its timing mode and parses its launcher-style line.
+    Must run before this process initialises the GPU. Returns the dropin_graph_predict object (value None with a reason when unavailable)."""
+    import re
+    import subprocess
+
+    exe = os.path.join(os.path.dirname(os.path.abspath(__file__)), "oracle", "_ref", "dropin_graph")
+    what = "Graph::predict + Context::synchronize of the reference's own graph code on Device::cuda(0) = this backend (three calls per 3x3 layer)"
+    if not os.path.exists(exe):
+        return {"value": None, "unit": "positions/sec", "what": what, "skipped": "oracle/_ref/dropin_graph is not built (make -C oracle dropin)"}
+    cmd = [exe, "time", str(batch), str(channels), str(blocks), "fp16" if dtype == "float16" else "fp32", "%g" % seconds, "3"]
+    try:
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60 + 4 * seconds)
+    except subprocess.TimeoutExpired:
+        return {"value": None, "unit": "positions/sec", "what": what, "skipped": "timed out"}
+    m = re.search(r"time = ([0-9.]+)s, repeats = (\d+), n/s = ([0-9.]+), ms per predict = ([0-9.]+)", res.stdout)
+    if res.returncode != 0 or m is None:
+        return {"value": None, "unit": "positions/sec", "what": what, "skipped": "exit code %d: %s" % (res.returncode, res.stdout[-300:])}
+    return {"value": float(m.group(3)), "unit": "positions/sec", "ms_per_step": float(m.group(4)), "repeats": int(m.group(2)),
+            "seconds": float(m.group(1)), "what": what}
+
+
+def timed_passes(ctx, forward, steps, warmup):
+    """Seconds per pass: `warmup` untimed passes, then `steps` passes between two synchronisations of the context's stream."""
+    for _ in range(warmup):
+        forward()
+    ctx.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        forward()
+    ctx.synchronize()
+    return (time.perf_counter() - t0) / steps
 
 def measured_gemm_traffic_bytes(config):
     """HBM bytes of one launch of the block-convolution GEMM kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (two runs, each counter
@@ -171,6 +216,13 @@ def run_int8(args, ml):
                      + " (3x3 convolution as implicit GEMM, M=%d N=%d K=%d)" % (pix, channels, 9 * channels),
                      "algorithmic_ops": conv_ops, "algorithmic_bytes": conv_bytes, "launches_timed": count, "avg_launch_us": t_conv * 1e6},
     }
+    if not args.unfused:
+        # the reference's route for an int8 layer on a device: im2row -> int8 GEMM into int32 -> requantisation (src/layers/Conv2D.cpp:214-239)
+        three = QuantizedResNet(ctx, batch, board, planes, channels, blocks, params, ranges, "reference")
+        three.setInput(x)
+        t3 = timed_passes(ctx, three.forward, args.steps, args.warmup)
+        result["reference_call_sequence"] = {"value": batch / t3, "unit": "positions/sec", "ms_per_step": 1e3 * t3,
+                                             "what": "im2row, int8 GEMM (gemm_v2 into int32) and quantized_scale_shift_act as three calls per layer"}
     if args.cpu_seconds > 0:
         result["cpu_baseline"] = run_int8_cpu_baseline(net.host_parameters, blocks, Q.quantize_tensor(x, net.transforms[0]), args.cpu_seconds)
     print(json.dumps(result))
@@ -264,6 +316,99 @@ def run_hybrid(args, ml):
     print(json.dumps(result))
 
 
+def run_conv_sweep(args, ml):
+    """Configuration 4: hip_convolution_implicit_gemm_forward on 19x19 boards, batch 512, fp16, N(0,1) inputs, He-normal weights, with bias,
+    residual and ReLU in the kernel's epilogue, for 64 / 128 / 256 / 384 channels and kernels 1 / 3 / 5. A step is the 12 layers one after
+    the other. Every row is priced with its algorithmic work (2 * M * C * C * k * k flops; input, residual and output once, weights and bias
+    once) against whichever of HBM and the fp16 MFMA peak bounds it; the top-level roofline object is the row that takes longest."""
+    batch, board = args.batch or 512, 19
+    pix = batch * board * board
+    rng = np.random.default_rng(3)
+    half = lambda a: np.ascontiguousarray(a, np.float32).astype(np.float16).view(np.uint16)
+    ctx = ml.Context(0)
+    layers = []
+    host = {}
+    for chans in (64, 128, 256, 384):
+        xh = half(rng.standard_normal((batch, board, board, chans), dtype=np.float32))
+        rh = half(rng.standard_normal((batch, board, board, chans), dtype=np.float32))
+        bh = half(rng.standard_normal(chans, dtype=np.float32) * 0.1)
+        x, res, bias = ml.toDevice(ctx, xh, "float16"), ml.toDevice(ctx, rh, "float16"), ml.toDevice(ctx, bh, "float16")
+        y = ml.Tensor((batch, board, board, chans), "float16")
+        for k in (1, 3, 5):
+            wh = half(rng.standard_normal((chans, k, k, chans), dtype=np.float32) * np.sqrt(2.0 / (k * k * chans)))
+            layers.append((chans, k, x, ml.toDevice(ctx, wh, "float16"), y, bias, res))
+            host[(chans, k)] = (xh, wh, bh, rh)
+
+    def step():
+        for chans, k, x, w, y, bias, res in layers:
+            ml.set_timer_label("C%d_k%d" % (chans, k))
+            ml.convolutionImplicitGemmForward(ctx, x, w, y, bias, res, "relu")
+        ml.set_timer_label(None)
+
+    t_step = timed_passes(ctx, step, args.steps, args.warmup)
+    timer = ml.KernelTimer(ctx)
+    ml.set_kernel_timer(timer)
+    for _ in range(max(1, min(args.steps, 5))):
+        step()
+    kernels = timer.summary()
+    ml.set_kernel_timer(None)
+    rows = []
+    for chans, k, *_ in layers:
+        n, t = kernels["convolution_implicit_gemm_forward@C%d_k%d" % (chans, k)]
+        flops = 2.0 * pix * chans * chans * k * k
+        nbytes = 2.0 * (3 * pix * chans + k * k * chans * chans + chans)
+        hbm = nbytes / (PEAK_HBM_GBS * 1e9) >= flops / (PEAK_MFMA_TFLOPS["float16"] * 1e12)
+        achieved = nbytes / t / 1e9 if hbm else flops / t / 1e12
+        peak = PEAK_HBM_GBS if hbm else PEAK_MFMA_TFLOPS["float16"]
+        rows.append({"channels": chans, "kernel_size": k, "avg_launch_us": t * 1e6, "launches_timed": n, "bound": "hbm" if hbm else "mfma",
+                     "achieved": achieved, "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s", "frac": achieved / peak,
+                     "algorithmic_bytes": nbytes, "algorithmic_flops": flops})
+    slowest = max(rows, key=lambda r: r["avg_launch_us"])
+    total_flops = sum(r["algorithmic_flops"] for r in rows)
+    result = {
+        "metric": "positions/sec (%s)" % CONV_SWEEP, "value": batch / t_step, "unit": "positions/sec", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": 1e3 * t_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic (N(0,1) inputs and residuals, He-normal weights, N(0,0.1) biases, seed 3)",
+        "config": {"workload": CONV_SWEEP, "batch": batch, "board": board, "channels": [64, 128, 256, 384], "kernel_sizes": [1, 3, 5],
+                   "epilogue": "bias + residual + ReLU inside the convolution kernel", "step": "the 12 layers one after the other"},
+        "tflops_executed": total_flops / t_step / 1e12,
+        "roofline": {"bound": slowest["bound"], "achieved": slowest["achieved"], "peak": slowest["peak"], "unit": slowest["unit"], "frac": slowest["frac"],
+                     "traffic": None, "kernel": "kernel_gemm_dma<fp16, im2row, bias + residual + ReLU> (C=%d, k=%d: M=%d N=%d K=%d)"
+                     % (slowest["channels"], slowest["kernel_size"], pix, slowest["channels"], slowest["kernel_size"] ** 2 * slowest["channels"]),
+                     "algorithmic_flops": slowest["algorithmic_flops"], "algorithmic_bytes": slowest["algorithmic_bytes"],
+                     "launches_timed": slowest["launches_timed"], "avg_launch_us": slowest["avg_launch_us"]},
+        "rows": rows,
+    }
+    if args.cpu_seconds > 0:
+        import oracle as O
+
+        ref = O.reference()
+        if ref is not None:
+            kind, cores, conv = "reference", 1, ref.conv2d_forward
+        else:
+            cores = min(16, os.cpu_count() or 1)
+            O.set_num_threads(cores)
+            kind, conv = "port", O.conv2d_forward
+
+        def cpu_step(positions):
+            t0 = time.perf_counter()
+            for (chans, k), (xh, wh, bh, rh) in host.items():
+                conv(xh[:positions], wh, bh, rh[:positions], O.RELU)
+            return time.perf_counter() - t0
+
+        positions = 1
+        t = cpu_step(positions)
+        # at most 192 positions: the reference counts the bytes of the im2row matrix (positions x 361 x 25 x 384 halfs) in 32-bit integers
+        target = int(max(1, min(batch, 192, args.cpu_seconds / max(t, 1e-9))))
+        if target > positions:
+            positions = target
+            t = cpu_step(positions)
+        result["cpu_baseline"] = {"value": positions / t, "unit": "positions/sec", "cores": cores, "kind": kind,
+                                  "sample": "%d positions through the same 12 layers (im2row + gemm_ex with the fused epilogue, the reference's "
+                                            "explicit-GEMM convolution), %.1f s" % (positions, t)}
+    print(json.dumps(result))
+
+
 def copy_calibration(ml, ctx):
     """One copy kernel of known size (256 MiB read, 256 MiB written) so that a counter run can be scaled against it."""
     n = 128 * 1024 * 1024
@@ -278,11 +423,16 @@ def copy_calibration(ml, ctx):
 
 
 def main():
+    import faulthandler
+
+    faulthandler.enable()
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--config", default="cfg2_resnet20x256_fp16_b1024", choices=sorted(CONFIGS))
+    ap.add_argument("--config", default="cfg2_resnet20x256_fp16_b1024", choices=sorted(CONFIGS) + [CONV_SWEEP])
+    ap.add_argument("--dropin-seconds", type=float, default=3.0,
+                    help="seconds the reference's own Graph is timed on this backend in a child process (0 disables; residual-network configurations)")
     ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments only; the metric is quoted at the default)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
@@ -297,9 +447,17 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    dropin = None
+    if args.config != CONV_SWEEP and CONFIGS[args.config][5] in ("float16", "float32") and args.dropin_seconds > 0 and not args.chunk:
+        # first of all: the child process has the device to itself, and this process has not touched the GPU yet
+        b, _, _, c, n, d, _ = CONFIGS[args.config]
+        dropin = run_dropin_graph(args.batch or b, c, n, d, args.dropin_seconds)
+
     from minml_amd import core as ml
     from minml_amd.resnet import ResNet, make_input, make_parameters, DEFAULT_CHUNK
 
+    if args.config == CONV_SWEEP:
+        return run_conv_sweep(args, ml)
     if CONFIGS[args.config][5] == "int8":
         return run_int8(args, ml)
     if CONFIGS[args.config][5] in ("hybrid", "hybrid_moe"):
@@ -394,6 +552,13 @@ def main():
                       "hbm_limited_ceiling_frac": min(1.0, gemm_flops / gemm_bytes * PEAK_HBM_GBS * 1e9 / (PEAK_MFMA_TFLOPS[dtype] * 1e12))},
         "transforms": transforms,
     }
+    if not args.unfused:
+        t3 = timed_passes(ctx, lambda: net.forward(fused=False), args.steps, args.warmup)
+        result["reference_call_sequence"] = {"value": batch / t3, "unit": "positions/sec", "ms_per_step": 1e3 * t3,
+                                             "what": "winograd_input_transform, gemm_batched_v2 and winograd_output_transform as three calls per 3x3 layer, "
+                                                     "as src/layers/Conv2D.cpp:365-378 issues them; same results bit for bit"}
+    if dropin is not None:
+        result["dropin_graph_predict"] = dropin
     if args.cpu_seconds > 0:
         params_storage = [(to_storage(w), to_storage(b)) for (w, b) in params]
         result["cpu_baseline"] = run_cpu_baseline(params_storage, to_storage(x), blocks, args.cpu_seconds)

@@ -140,7 +140,9 @@ extern "C"
 	 * HIP graph capture, serving loops and harnesses that forbid hipMalloc. hip_winograd_layer_forward keeps the counters and the
 	 * product scratch of its one-launch form in the context's growable workspace (hipMalloc on first use); this entry point keeps them in
 	 * a static device array of the library (18.1 MiB per GPU, held until the process ends) and clears its counters with a kernel. Limit:
-	 * at most 4096 images per call (larger batches are rejected with std::logic_error: split them). All calls on one GPU share that
+	 * at most 4096 images per call at the shape that uses the array (256 -> 256 channels, 16 tiles per image, fp16, 256 CUs; larger
+	 * batches of it are rejected with std::logic_error: split them); every other shape runs as the batched product followed by the fused
+	 * transform, which use no library-side memory at all and take any batch. All calls on one GPU share that
 	 * array: calls that overlap on one GPU (two contexts, two threads) race; calls on one context run in stream order and are safe.
 	 */
 	void hip_winograd_layer_forward_static(mlContext_t context, int tile_size, const mlTensor_t input_matrices, const mlTensor_t weight_matrices,
@@ -217,7 +219,9 @@ extern "C"
 	void hip_moe_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t w, const mlTensor_t b, float beta, mlTensor_t y,
 			mlActivationType_t act); /* y [B, K, E, N] = act(x [B, K, E, C] . w[e] [N, C]^T + b [E, N] + beta * y), one dense layer per expert (moe.cu:1395-1432) */
 	void hip_scatter_tokens_forward(mlContext_t context, const mlTensor_t x, const mlTensor_t indices_and_values, float beta,
-			mlTensor_t y); /* y [B, H, W, C] = beta * y + sum over the slots holding each token of gate * x [B, K, E, C], in fp32, experts ascending (moe.cu:559-582) */
+			mlTensor_t y); /* y [B, H, W, C] = beta * y + sum over the slots holding each token of gate * x [B, K, E, C], in fp32, experts ascending (moe.cu:559-582).
+			                * A token may hold at most one slot per expert, as every router of this library and of the reference writes its table; of
+			                * duplicates in a hand-made table only the lowest slot counts, where the reference's atomic additions would add them all. */
 
 	/* ---- additions with no counterpart in the reference ABI ----
 	 * hip_quantized_conv_forward: the whole int8 convolution of reference src/layers/Conv2D.cpp:240-308 (int8 implicit GEMM with

@@ -166,6 +166,10 @@ def fn(name):
         flag = _error_flag
 
         def wrapped(*args):
+            if flag.value != 0:  # left behind by a raw call that went round this wrapper: report it as what it is, not as this call's failure
+                _lib.hip_take_last_error(_error_buffer, 2048)
+                raise RuntimeError("an earlier call into the library failed and its error was never collected: %s"
+                                   % _error_buffer.value.decode("utf-8", "replace"))
             result = raw(*args)
             if flag.value != 0:
                 check_error()

@@ -79,17 +79,39 @@ class Graph:
         B.fn("graph_begin_capture")(context.handle)
         try:
             function()
-        finally:
-            handle = B.fn("graph_end_capture")(context.handle)
-        return Graph(context, handle)
+        except BaseException:
+            # the recording must be closed whatever happened; what it produced is dropped, and the caller sees the original failure
+            try:
+                handle = B.fn("graph_end_capture")(context.handle)
+                if handle:
+                    B.fn("graph_destroy")(handle)
+            except Exception:
+                pass
+            raise
+        return Graph(context, B.fn("graph_end_capture")(context.handle))
 
     def launch(self):
+        if not self.handle:
+            raise RuntimeError("the graph was destroyed")
         B.fn("graph_launch")(self.context.handle, self.handle)
 
     def destroy(self):
         if self.handle:
-            B.fn("graph_destroy")(self.handle)
-            self.handle = None
+            handle, self.handle = self.handle, None
+            B.fn("graph_destroy")(handle)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.destroy()
+        return False
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:  # interpreter shutdown: the library may be gone already
+            pass
 
 
 class Event:

@@ -39,6 +39,26 @@ namespace mlhip
 	 * is a function-try-block whose handler calls entry_failed; with capture off the handler rethrows and nothing changes.
 	 */
 	bool capture_current_exception(); /* runtime.hip; call from a catch handler only */
+	/*
+	 * Some entry points are written in terms of others (gemm_v2 -> gemm, winograd_layer_forward -> gemm_batched + fused transform ...).
+	 * Such a function holds a NestedEntryCalls object while it calls them: as long as one exists on the calling thread, an inner entry
+	 * point never captures — its handler rethrows, the exception unwinds to the outermost function-try-block (whose handler runs after
+	 * the object is gone) and is captured there, so a failed outer call has launched nothing after the failure.
+	 */
+	int& nested_entry_depth(); /* runtime.hip; thread-local */
+	struct NestedEntryCalls
+	{
+			NestedEntryCalls()
+			{
+				++nested_entry_depth();
+			}
+			~NestedEntryCalls()
+			{
+				--nested_entry_depth();
+			}
+			NestedEntryCalls(const NestedEntryCalls&) = delete;
+			NestedEntryCalls& operator=(const NestedEntryCalls&) = delete;
+	};
 	template<typename R>
 	inline R entry_failed()
 	{
@@ -77,6 +97,9 @@ namespace mlhip
 	}
 	/* returns device scratch of at least `bytes` bytes; grows by reallocating after the stream has drained */
 	void* get_workspace(mlContext_t context, size_t bytes);
+	/* winograd.hip; called once per context creation with that device current: looks up, per device, the address of the static device
+	 * array behind hip_winograd_layer_forward_static and raises the dynamic-LDS limit of the kernels that run from it */
+	void prepare_static_memory(int device_index);
 	/* number of compute units of the current device (cached per device) */
 	int device_compute_units();
 	/* makes sure a kernel may be launched with `bytes` of dynamic LDS on the current device (requests above the 64 KB default raise the

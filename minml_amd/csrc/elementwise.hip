@@ -260,6 +260,7 @@ extern "C"
 		if (volume(x) == 0)
 			return;
 		MLHIP_REQUIRE(x.dtype == y.dtype && volume(x) == volume(y), "activation_forward: x and y must have one shape and data type");
+		mlhip::NestedEntryCalls nested;
 		if (act == ACTIVATION_LINEAR)
 		{ /* the reference copies and ignores alpha / beta in this case */
 			if (x.data != y.data)
@@ -307,12 +308,18 @@ extern "C"
 		return mlhip::entry_failed<void>();
 	}
 	void hip_scale_tensor(mlContext_t context, float alpha, mlTensor_t x)
+	try
 	{ /* x *= alpha (reference: src/backend/cuda/kernels/tensor_op.cu:318-321) */
+		mlhip::NestedEntryCalls nested;
 		mlTensor_t none;
 		none.data = nullptr;
 		none.dtype = x.dtype;
 		none.rank = 0;
 		hip_add_tensors(context, 0.0f, none, 0.0f, none, 0.0f, none, alpha, x);
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
 	}
 	void hip_convert_type(mlContext_t context, void *dst, mlDataType_t dst_dtype, const void *src, mlDataType_t src_dtype, int elements)
 	try
@@ -320,6 +327,7 @@ extern "C"
 		if (elements <= 0)
 			return;
 		MLHIP_REQUIRE(dst != nullptr && src != nullptr, "convert_type: null pointer");
+		mlhip::NestedEntryCalls nested;
 		if (dst_dtype == src_dtype)
 		{
 			if (dst != src)

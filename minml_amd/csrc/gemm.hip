@@ -377,6 +377,7 @@ extern "C"
 		}
 		else
 			MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm: A, B and C must have one data type");
+		mlhip::NestedEntryCalls nested;
 		hip_gemm(context, dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
 	}
 	catch (...)
@@ -388,6 +389,7 @@ extern "C"
 	{
 		MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype, "gemm_batched: A, B and C must have one data type");
 		MLHIP_REQUIRE(C.dtype == DTYPE_FLOAT16 || C.dtype == DTYPE_FLOAT32, "gemm_batched: unsupported data type");
+		mlhip::NestedEntryCalls nested;
 		hip_gemm_batched(context, C.dtype, shape_of(C), C.data, shape_of(A), A.data, shape_of(B), B.data, opA, opB, alpha, beta);
 	}
 	catch (...)

@@ -286,7 +286,7 @@ namespace
 				for (int i = 0; i < GROUP; i++)
 				{
 					const unsigned long long hits = __ballot(k0 + lane < capacity && e0 + i < experts && index[i] == token);
-					if (hits != 0ull) /* at most one slot per expert holds the token */
+					if (hits != 0ull && found[i] < 0) /* a token holds at most one slot per expert; of duplicates in a hand-made table the lowest counts */
 						found[i] = k0 + __builtin_ctzll(hits);
 				}
 			}

@@ -161,12 +161,20 @@ namespace mlhip
 	{
 		std::atomic<int> error_capture { 0 };
 		std::mutex error_mutex;
-		int error_kind = 0; /* 0 none, 1 std::logic_error, 2 std::runtime_error or another std::exception, 3 anything else */
+		/* 0 none, 1 std::logic_error, 2 std::runtime_error or another std::exception, 3 anything else; written under the mutex, read by
+		 * hosts through hip_error_flag_address without it, hence atomic */
+		std::atomic<int> error_kind { 0 };
+		static_assert(sizeof(std::atomic<int>) == sizeof(int) && std::atomic<int>::is_always_lock_free, "the error flag is exposed as a plain int");
 		std::string error_message;
+	}
+	int& nested_entry_depth()
+	{
+		thread_local int depth = 0;
+		return depth;
 	}
 	bool capture_current_exception()
 	{
-		if (error_capture.load() == 0)
+		if (error_capture.load() == 0 || nested_entry_depth() > 0)
 			return false;
 		int kind = 3;
 		std::string message = "unknown exception";
@@ -188,10 +196,10 @@ namespace mlhip
 		{
 		}
 		std::lock_guard<std::mutex> lock(error_mutex);
-		if (error_kind == 0)
+		if (error_kind.load() == 0)
 		{ /* the first failure since the last hip_take_last_error is the one reported */
-			error_kind = kind;
 			error_message = message;
+			error_kind.store(kind);
 		}
 		return true;
 	}
@@ -205,19 +213,19 @@ extern "C"
 	}
 	const int* hip_error_flag_address(void)
 	{
-		return &mlhip::error_kind;
+		return reinterpret_cast<const int*>(&mlhip::error_kind);
 	}
 	int hip_take_last_error(char *buffer, int size)
 	{
 		std::lock_guard<std::mutex> lock(mlhip::error_mutex);
-		const int kind = mlhip::error_kind;
+		const int kind = mlhip::error_kind.load();
 		if (buffer != nullptr && size > 0)
 		{
 			const size_t n = std::min(static_cast<size_t>(size - 1), mlhip::error_message.size());
 			std::memcpy(buffer, mlhip::error_message.data(), n);
 			buffer[n] = 0;
 		}
-		mlhip::error_kind = 0;
+		mlhip::error_kind.store(0);
 		mlhip::error_message.clear();
 		return kind;
 	}
@@ -307,6 +315,9 @@ extern "C"
 		ctx->device_index = device_index;
 		/* a blocking stream, as in the reference (src/backend/cuda/utils.cpp:115): context-less (synchronous) copies order against it */
 		MLHIP_CHECK(hipStreamCreate(&ctx->stream));
+		/* set-up that entry points must not do on their first call (a caller may be recording a graph by then): the device address of the
+		 * library's static device memory and the LDS limits of the kernels that use it */
+		prepare_static_memory(device_index);
 		return ctx;
 	}
 	catch (...)
@@ -416,7 +427,11 @@ extern "C"
 	try
 	{
 		MLHIP_REQUIRE(graph != nullptr, "hip_graph_launch: null graph");
-		MLHIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, stream_of(context)));
+		Context *ctx = get(context);
+		MLHIP_REQUIRE(reinterpret_cast<Graph*>(graph)->device_index == ctx->device_index,
+				"hip_graph_launch: the graph was recorded on another device than the context's");
+		use_device(ctx->device_index);
+		MLHIP_CHECK(hipGraphLaunch(reinterpret_cast<Graph*>(graph)->exec, ctx->stream));
 	}
 	catch (...)
 	{

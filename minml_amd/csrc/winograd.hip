@@ -1131,16 +1131,22 @@ namespace
 		for (unsigned int i = blockIdx.x * blockDim.x + threadIdx.x; i < words; i += gridDim.x * blockDim.x)
 			dst[i] = 0u;
 	}
-	bool layer_kernel_applies(const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlShape_t &shape, const mlTensor_t &bias,
+	/* the shapes the one-launch kernel is written for, the upper limit of the batch (layer_batch_fits) apart */
+	bool layer_kernel_shape(const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlShape_t &shape, const mlTensor_t &bias,
 			const mlTensor_t &ext, const void *output, mlActivationType_t act)
 	{
 		const auto aligned16 = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) % 16) == 0; };
 		return input_matrices.dtype == DTYPE_FLOAT16 && shape.dim[3] == LAYER_CHANNELS && input_matrices.dim[2] == LAYER_CHANNELS
 				&& weight_matrices.dim[1] == LAYER_CHANNELS && weight_matrices.dim[2] == LAYER_CHANNELS
 				&& ceil_div(shape.dim[1], 4) * ceil_div(shape.dim[2], 4) == 16 && shape.dim[0] % 4 == 0 && shape.dim[0] >= 4 * LAYER_XCDS
-				&& shape.dim[0] <= 4 * LAYER_XCDS * LAYER_MAX_CHUNKS && (act == ACTIVATION_LINEAR || act == ACTIVATION_RELU)
+				&& (act == ACTIVATION_LINEAR || act == ACTIVATION_RELU)
 				&& aligned16(input_matrices.data) && aligned16(weight_matrices.data) && aligned16(bias.data) && aligned16(ext.data) && aligned16(output)
 				&& device_compute_units() == 256;
+	}
+	/* the per-XCD counters (in the workspace or in the static array) cover this many images per launch */
+	bool layer_batch_fits(const mlShape_t &shape)
+	{
+		return shape.dim[0] <= 4 * LAYER_XCDS * LAYER_MAX_CHUNKS;
 	}
 	void launch_layer(mlContext_t context, const mlTensor_t &input_matrices, const mlTensor_t &weight_matrices, const mlTensor_t &bias, const mlTensor_t &ext,
 			const mlShape_t &shape, void *output, mlActivationType_t act, mlTensor_t &next, bool static_memory)
@@ -1184,6 +1190,14 @@ namespace
 		}
 #undef MLHIP_LAUNCH_LAYER
 		MLHIP_CHECK(hipGetLastError());
+	}
+}
+
+namespace mlhip
+{
+	void prepare_static_memory(int device_index)
+	{
+		(void) layer_static_pointer(device_index);
 	}
 }
 
@@ -1297,6 +1311,7 @@ extern "C"
 		{ /* shapes the fused kernel does not take: the two stand-alone transforms, which need y in memory */
 			MLHIP_REQUIRE(output != nullptr, "Winograd fused transform: this shape needs the output tensor as intermediate storage");
 			mlTensor_t y = make_tensor(output, matrices.dtype, output_shape);
+			mlhip::NestedEntryCalls nested;
 			hip_winograd_output_transform(context, tile_size, matrices, bias, ext, y, act);
 			hip_winograd_input_transform(context, tile_size, y, next_matrices);
 			return;
@@ -1333,19 +1348,23 @@ extern "C"
 			MLHIP_REQUIRE(bias.dtype == input_matrices.dtype && volume(bias) == static_cast<size_t>(output_shape.dim[3]), "Winograd layer: bias must be [Cout]");
 		if (ext.data != nullptr)
 			MLHIP_REQUIRE(ext.dtype == input_matrices.dtype && volume(ext) == volume(output_shape), "Winograd layer: ext must have the output's shape and dtype");
-		if (layer_kernel_applies(input_matrices, weight_matrices, output_shape, bias, ext, output, act))
+		if (layer_kernel_shape(input_matrices, weight_matrices, output_shape, bias, ext, output, act))
 		{
-			mlTensor_t next = next_matrices;
-			launch_layer(context, input_matrices, weight_matrices, bias, ext, output_shape, output, act, next, static_memory);
-			return;
+			if (layer_batch_fits(output_shape))
+			{
+				mlTensor_t next = next_matrices;
+				launch_layer(context, input_matrices, weight_matrices, bias, ext, output_shape, output, act, next, static_memory);
+				return;
+			}
+			/* the one shape whose launch uses the library's static memory: a batch beyond what that memory covers is refused, not rerouted */
+			MLHIP_REQUIRE(!static_memory, "Winograd layer (static memory): at most 4096 images per call fit the library's static counters; split the batch");
 		}
-		if (static_memory)
-			MLHIP_REQUIRE(output_shape.dim[0] <= 4 * LAYER_XCDS * LAYER_MAX_CHUNKS,
-					"Winograd layer (static memory): at most 4096 images per call fit the library's static counters; split the batch");
-		/* every other shape: the batched product into the caller's matrices, then the fused (or two-step) transform */
+		/* every other shape: the batched product into the caller's matrices, then the fused (or two-step) transform; neither uses
+		 * library-side memory, so the static entry point takes these shapes at any batch size */
 		MLHIP_REQUIRE(output_matrices.data != nullptr && output_matrices.dtype == input_matrices.dtype && output_matrices.rank == 3
 				&& output_matrices.dim[0] == 36 && static_cast<size_t>(output_matrices.dim[1]) == tiles && output_matrices.dim[2] == output_shape.dim[3],
 				"Winograd layer: this shape needs output matrices [36, tiles, Cout] as intermediate storage");
+		mlhip::NestedEntryCalls nested;
 		hip_gemm_batched(context, input_matrices.dtype, shape_of(output_matrices), output_matrices.data, shape_of(input_matrices), input_matrices.data,
 				shape_of(weight_matrices), weight_matrices.data, 'n', 't', 1.0f, 0.0f);
 		hip_winograd_output_input_transform(context, tile_size, output_matrices, bias, ext, output_shape, output, act, next_matrices);

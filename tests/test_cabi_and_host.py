@@ -194,6 +194,10 @@ def test_library_errors_surface_as_python_exceptions():
         B.fn("winograd_input_transform")(None, 3, desc, B.make_tensor(1, B.DTYPE_FLOAT32, (36, 1, 4)))
     with pytest.raises(ValueError, match="matrix op"):
         B.fn("gemm_v2")(None, b"x", b"n", 1.0, desc, desc, 0.0, desc)
+    # entry points written in terms of others (gemm_v2 above; scale_tensor -> add_tensors here): the inner failure unwinds to the outermost
+    # call and is reported once, as that call's failure
+    with pytest.raises(ValueError, match="add_tensors: unsupported data type"):
+        B.fn("scale_tensor")(None, 2.0, B.make_tensor(1, B.DTYPE_INT32, (8,)))
     # the failure was taken: the next call starts clean, and one that succeeds raises nothing
     assert B.fn("take_last_error")(None, 0) == 0
     assert B.fn("get_number_of_devices")() >= 0
