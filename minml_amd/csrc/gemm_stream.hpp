@@ -4,13 +4,14 @@
  *
  * This product is bound by HBM, not by the matrix cores: one matrix pair moves T*512 bytes in and T*N*s bytes out for only
  * 2*T*N*K flops, and the 36 B operands together are a few megabytes. The kernel is therefore organised around the A stream:
- *   - persistent workgroups (one per CU), each owning a contiguous range of "units" (128 rows of A of one matrix) and, with 8
+ *   - persistent workgroups (one per CU), each owning a set of "units" (128 rows of A of one matrix; 64 rows for the plain batched
+ *     products on the 8-wavefront layout, see launch_stream_gemm_as) and, with 8
  *     wavefronts of 32 columns each, all 256 columns of N, so that every row of A is fetched by exactly one workgroup (for wider N the
  *     column slices of one row range sit on one XCD and share its L2);
  *   - every wavefront keeps ITS part of the B operand (32 columns x full K = 64 VGPRs) in registers for the whole run of units that
  *     share a matrix, so B costs neither LDS space nor LDS bandwidth;
  *   - A moves HBM -> LDS with direct-to-LDS loads (global_load_lds_dwordx4, no staging registers) into a ring of 128-byte-per-row
- *     stages that runs ahead across unit boundaries (STAGES - 1 stages of 16 KB), so loads never stop for an epilogue or for the next
+ *     stages that runs ahead across unit boundaries (STAGES - 1 stages of 16 KB, or of 8 KB for units of 64 rows), so loads never stop for an epilogue or for the next
  *     unit's prologue; completion is tracked with explicit vmcnt waits and fence-free barriers (a fence would drain the whole ring);
  *   - two wavefronts per SIMD: one that waits (full memory pipeline, stage barrier, store epilogue) leaves the SIMD to the other;
  *   - fragment reads of k step t + 1 are in flight while k step t is multiplied (register double buffer);
@@ -60,36 +61,18 @@ namespace mlhip
 			static constexpr int STAGES_PER_UNIT = K_BYTES / STAGE_K_BYTES; /* 4 */
 	};
 
-	/* at most `stages` stages of LOADS vector-memory operations each may remain outstanding */
-	template<int LOADS>
+	/* at most `stages` stages of LOADS vector-memory operations each may remain outstanding (stages <= MAX; the counter holds up to 63) */
+	template<int LOADS, int MAX = 14>
 	__device__ __forceinline__ void wait_vmcnt_stages(int stages)
 	{
-		switch (stages)
+		if constexpr (MAX == 0)
+			wait_vmcnt<0>();
+		else
 		{
-			case 0:
-				wait_vmcnt<0>();
-				break;
-			case 1:
-				wait_vmcnt<LOADS>();
-				break;
-			case 2:
-				wait_vmcnt<2 * LOADS>();
-				break;
-			case 3:
-				wait_vmcnt<3 * LOADS>();
-				break;
-			case 4:
-				wait_vmcnt<4 * LOADS>();
-				break;
-			case 5:
-				wait_vmcnt<5 * LOADS>();
-				break;
-			case 6:
-				wait_vmcnt<6 * LOADS>();
-				break;
-			default:
-				wait_vmcnt<7 * LOADS>();
-				break;
+			if (stages >= MAX)
+				wait_vmcnt<(MAX * LOADS <= 63) ? MAX * LOADS : 63>();
+			else
+				wait_vmcnt_stages<LOADS, MAX - 1>(stages);
 		}
 	}
 	template<int N, typename F>
@@ -128,7 +111,7 @@ namespace mlhip
 	 * matrix of the batch. Consecutive rows of A lie a_row_bytes apart (KB for a dense matrix; more when the matrices of the batch are
 	 * interleaved row by row, as the experts' tokens are).
 	 */
-	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue>
+	template<typename T, int KB, int WAVES_M, int WAVES_N, int STAGES, typename Epilogue, int BM = StreamGemmConfig::BM>
 	__global__ __launch_bounds__(64 * WAVES_M * WAVES_N, 1) void kernel_gemm_stream_wide_nt(const T *A, const T *B, T *C, int M, int N, size_t stride_a,
 			size_t stride_b, size_t stride_c, int batch, int tiles_m, int n_tiles, int units_per_group, int sweep, size_t a_row_bytes, Epilogue epilogue)
 	{
@@ -140,18 +123,19 @@ namespace mlhip
 		constexpr bool PACKED = stream_epilogue_reads_nothing<Epilogue>::value;
 		constexpr int WAVES = WAVES_M * WAVES_N;
 		constexpr int BN = 32 * WAVES_N;
-		constexpr int ROWS = Cfg::BM / WAVES_M; /* rows of a unit owned by one wavefront */
+		constexpr int STAGE_BYTES = BM * Cfg::STAGE_K_BYTES; /* one stage: 128 bytes of K of every row of a unit */
+		constexpr int ROWS = BM / WAVES_M; /* rows of a unit owned by one wavefront */
 		constexpr int BLOCKS = ROWS / 32;
 		constexpr int STAGES_PER_UNIT = KB / Cfg::STAGE_K_BYTES;
 		constexpr int DISTANCE = STAGES - 1; /* stages requested ahead of the one being multiplied */
-		constexpr int LOADS = 16 / WAVES; /* 1 KB blocks of a 16 KB stage moved by one wavefront */
+		constexpr int LOADS = (STAGE_BYTES / 1024) / WAVES; /* 1 KB blocks of a stage moved by one wavefront */
 		constexpr int SLAB_STRIDE = 32 * (PACKED ? sizeof(T) : 4) + 16;
 		constexpr int KSTEPS = 4; /* MFMA k steps per stage */
 		static_assert(KB % Cfg::STAGE_K_BYTES == 0 && ROWS % 32 == 0, "unsupported unit shape");
-		static_assert(16 % WAVES == 0 && DISTANCE >= 2 && DISTANCE <= 8 && (DISTANCE - 2) * LOADS <= 63, "unsupported workgroup shape");
+		static_assert(LOADS >= 1 && (STAGE_BYTES / 1024) % WAVES == 0 && DISTANCE >= 2 && DISTANCE <= 16 && (DISTANCE - 2) * LOADS <= 63, "unsupported workgroup shape");
 		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 		uint8_t *ring = lds;
-		uint8_t *slab = lds + STAGES * Cfg::STAGE_BYTES + (threadIdx.x >> 6) * (32 * SLAB_STRIDE);
+		uint8_t *slab = lds + STAGES * STAGE_BYTES + (threadIdx.x >> 6) * (32 * SLAB_STRIDE);
 
 		const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 		const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
@@ -243,8 +227,8 @@ namespace mlhip
 			auto request_stage = [&](int g) __attribute__((always_inline))
 			{
 				const int u = g / STAGES_PER_UNIT, ks = g - u * STAGES_PER_UNIT;
-				const int m_first = (tile_base + u * tile_step) * Cfg::BM;
-				uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
+				const int m_first = (tile_base + u * tile_step) * BM;
+				uint8_t *stage = ring + (g % STAGES) * STAGE_BYTES;
 #pragma unroll
 				for (int i = 0; i < LOADS; i++)
 				{
@@ -256,7 +240,7 @@ namespace mlhip
 			uint4_t frags[2][BLOCKS];
 			auto read_fragments = [&](int g, int kk, uint4_t (&regs)[BLOCKS]) __attribute__((always_inline))
 			{
-				const uint8_t *stage = ring + (g % STAGES) * Cfg::STAGE_BYTES;
+				const uint8_t *stage = ring + (g % STAGES) * STAGE_BYTES;
 #pragma unroll
 				for (int i = 0; i < BLOCKS; i++)
 					regs[i] = *reinterpret_cast<const uint4_t*>(stage + (frag_first[i] ^ (kk * 32)));
@@ -297,7 +281,7 @@ namespace mlhip
 				{
 					if (!local.has_extra())
 						return;
-					const int m_first = (tile_base + u * tile_step) * Cfg::BM + wave_m * ROWS;
+					const int m_first = (tile_base + u * tile_step) * BM + wave_m * ROWS;
 #pragma unroll
 					for (int i = 0; i < BLOCKS; i++)
 #pragma unroll
@@ -321,7 +305,7 @@ namespace mlhip
 			auto store_unit = [&](int u) __attribute__((always_inline))
 			{
 				/* lane l, register r of block i: m = 32 i + l % 32, n = 8 (r / 4) + 4 (l / 32) + r % 4 */
-				const int m_first = (tile_base + u * tile_step) * Cfg::BM + wave_m * ROWS;
+				const int m_first = (tile_base + u * tile_step) * BM + wave_m * ROWS;
 				if constexpr (PACKED)
 				{
 					T *out_base;
@@ -508,20 +492,24 @@ namespace mlhip
 	{
 		return (element_size == 2) ? stream_gemm_half_applies(M, batch, k_bytes) : stream_gemm_applies(M, batch, k_bytes);
 	}
-	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue>
-	inline void launch_stream_gemm_as(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
+	/*
+	 * How one launch divides its row blocks ("units" of BM rows of one matrix) among the workgroups. The grid is `groups` row-range groups
+	 * x n_tiles column slices. Two ways to hand out units: contiguous (group j takes units [j * units_per_group, ...) of the concatenated
+	 * (matrix, row block) sequence, ascending, crossing into the next matrix where its range does), or the sweep form (sweep > 0 groups per
+	 * matrix, group j of a matrix takes that matrix's row blocks j, j + sweep, ... from the last to the first). `rows_of_busiest_group`
+	 * is what the launch waits for: the rows the group with most units multiplies.
+	 */
+	struct StreamGemmPlan
 	{
-		typedef StreamGemmConfig Cfg;
-		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
-		constexpr int WAVES = WAVES_M * WAVES_N;
-		constexpr int SLAB_BYTES = WAVES * 32 * (32 * (stream_epilogue_reads_nothing<Epilogue>::value ? sizeof(T) : 4) + 16);
-		constexpr int STAGES = (8 * Cfg::STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? 8 : 7;
-		constexpr int LDS = STAGES * Cfg::STAGE_BYTES + SLAB_BYTES;
-		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
-		auto kernel = kernel_gemm_stream_wide_nt<T, KB, WAVES_M, WAVES_N, STAGES, Epilogue>;
-		ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), LDS);
-		const int tiles_m = ceil_div(g.M, Cfg::BM), n_tiles = ceil_div(g.N, 32 * WAVES_N);
-		const int total_units = g.batch * tiles_m;
+			int bm, tiles_m, groups, units_per_group, sweep;
+			long long rows_of_busiest_group;
+	};
+	inline StreamGemmPlan plan_stream_gemm(int M, int batch, int n_tiles, int bm, bool allow_sweep)
+	{
+		StreamGemmPlan p;
+		p.bm = bm;
+		p.tiles_m = ceil_div(M, bm);
+		const int total_units = batch * p.tiles_m;
 		int groups = device_compute_units() / n_tiles;
 		if (groups >= 8)
 			groups -= groups % 8; /* keeps the grid a multiple of 8 * n_tiles so that the column slices of a group share an XCD */
@@ -529,25 +517,73 @@ namespace mlhip
 			groups = 1;
 		if (groups > total_units)
 			groups = total_units;
-		const int units_per_group = ceil_div(total_units, groups);
+		p.groups = groups;
+		p.units_per_group = ceil_div(total_units, groups);
+		p.sweep = 0;
+		p.rows_of_busiest_group = static_cast<long long>(p.units_per_group) * bm;
 		/*
 		 * Sweep form for batched products whose matrices each get at least two workgroups (the 36 Winograd matrices on 256 compute
 		 * units: 7 each, 252 workgroups): measured 1.3 % to 2.8 % more positions per second on the 20-block network than the
-		 * contiguous split, although it leaves 4 compute units idle, because the rows meet the last-level cache in the right order.
+		 * contiguous split of the same units, although it leaves 4 compute units idle, because the rows meet the last-level cache in
+		 * the right order.
 		 */
-		int sweep = 0;
-		if (n_tiles == 1 && g.batch > 1 && groups / g.batch >= 2)
+		if (allow_sweep && n_tiles == 1 && batch > 1 && groups / batch >= 2)
 		{
-			const int per_matrix = min(groups / g.batch, tiles_m);
-			if ((groups - per_matrix * g.batch) * 16 <= groups) /* only when at most 1 / 16 of the compute units stay idle */
+			const int per_matrix = min(groups / batch, p.tiles_m);
+			if ((groups - per_matrix * batch) * 16 <= groups) /* only when at most 1 / 16 of the compute units stay idle */
 			{
-				sweep = per_matrix;
-				groups = sweep * g.batch;
+				p.sweep = per_matrix;
+				p.groups = per_matrix * batch;
+				p.rows_of_busiest_group = static_cast<long long>(ceil_div(p.tiles_m, per_matrix)) * bm;
 			}
 		}
-		hipLaunchKernelGGL(kernel, dim3(groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
-				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, tiles_m, n_tiles, units_per_group, sweep,
+		return p;
+	}
+	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue, int BM>
+	inline void launch_stream_gemm_planned(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue, const StreamGemmPlan &plan)
+	{
+		typedef StreamGemmConfig Cfg;
+		constexpr int WAVES = WAVES_M * WAVES_N;
+		constexpr int SLAB_BYTES = WAVES * 32 * (32 * (stream_epilogue_reads_nothing<Epilogue>::value ? sizeof(T) : 4) + 16);
+		constexpr int STAGE_BYTES = BM * Cfg::STAGE_K_BYTES;
+		constexpr int RING_STAGES = 128 * 1024 / STAGE_BYTES; /* 128 KB of ring where the slabs leave room for it: 8 stages of 128 rows, 16 of 64 */
+		constexpr int STAGES = (RING_STAGES * STAGE_BYTES + SLAB_BYTES <= 160 * 1024) ? RING_STAGES : RING_STAGES - RING_STAGES / 8;
+		constexpr int LDS = STAGES * STAGE_BYTES + SLAB_BYTES;
+		static_assert(LDS <= 160 * 1024, "ring and slabs must fit the 160 KB of LDS");
+		auto kernel = kernel_gemm_stream_wide_nt<T, KB, WAVES_M, WAVES_N, STAGES, Epilogue, BM>;
+		ensure_dynamic_lds(reinterpret_cast<const void*>(kernel), LDS);
+		const int n_tiles = ceil_div(g.N, 32 * WAVES_N);
+		hipLaunchKernelGGL(kernel, dim3(plan.groups * n_tiles), dim3(64 * WAVES), LDS, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B),
+				reinterpret_cast<T*>(g.C), g.M, g.N, g.stride_a, g.stride_b, g.stride_c, g.batch, plan.tiles_m, n_tiles, plan.units_per_group, plan.sweep,
 				g.a_row_bytes != 0 ? g.a_row_bytes : static_cast<size_t>(KB), epilogue);
+	}
+	template<typename T, int KB, int WAVES_M, int WAVES_N, typename Epilogue>
+	inline void launch_stream_gemm_as(hipStream_t stream, const StreamGemmArgs &g, const Epilogue &epilogue)
+	{
+		constexpr bool PLAIN = std::is_same<Epilogue, PlainStore>::value;
+		const int n_tiles = ceil_div(g.N, 32 * WAVES_N);
+		const StreamGemmPlan wide = plan_stream_gemm(g.M, g.batch, n_tiles, 128, true);
+		/*
+		 * Units of 64 rows for the plain batched products on the 1 x 8 wavefront layout (a wavefront then owns two 32-row blocks instead
+		 * of four: 32 accumulator registers less, half as long an epilogue per unit, a ring of 16 stages of 8 KB), in the sweep form and
+		 * where the busiest workgroup gets no more rows than with units of 128. Measured on MI355X, stand-alone, 256 -> 256 channels in
+		 * fp16: 16384 tiles 132 -> 120 us, 12800 tiles 107 -> 92 us, 4096 tiles 40 -> 38 us; 20 x 256 network 99.9 k -> 102.4 k positions/s
+		 * on the same box. The 2 x 4 layout (64 < N <= 128, or N = 384 as three slices) would own a single 32-row block per wavefront and
+		 * measures slower with it (128 channels 45 -> 46 us, 384 channels 206 -> 227 us, fp32 at 128 channels 57 -> 63 us), and the
+		 * contiguous split of 64-row units, although it balances 36 x 16384 rows perfectly over 256 workgroups, loses the sweep's order
+		 * through the last-level cache (96.0 k positions/s). Products with an epilogue functor (1x1 convolutions, the experts' layers)
+		 * measured level with units of 64 rows and keep units of 128.
+		 */
+		if constexpr (PLAIN && WAVES_M == 1)
+		{
+			const StreamGemmPlan fine = plan_stream_gemm(g.M, g.batch, n_tiles, 64, true);
+			if (fine.sweep > 0 && fine.rows_of_busiest_group <= wide.rows_of_busiest_group)
+			{
+				launch_stream_gemm_planned<T, KB, WAVES_M, WAVES_N, Epilogue, 64>(stream, g, epilogue, fine);
+				return;
+			}
+		}
+		launch_stream_gemm_planned<T, KB, WAVES_M, WAVES_N, Epilogue, 128>(stream, g, epilogue, wide);
 	}
 	/* wavefront layout by output width: 8 x 32 columns for N > 128, 2 x 4 for N > 64, 4 x 2 below */
 	template<typename T, int KB, typename Epilogue>
