@@ -8,6 +8,9 @@ layer and the input transform of the next run as one launch (bit-identical resul
 layer). Prints ONE JSON line:
 
   value        positions / second over the timed steps (wall clock between two stream synchronisations)
+               the better of two ways of issuing the same pass: the whole batch on one stream, or its two halves on two streams of the
+               device (`config.execution` says which; `single_stream` and `two_streams` hold both); every per-kernel figure below comes from
+               the single-stream pass, where launches do not overlap
   roofline     the dominant kernel, the 36-way batched Winograd GEMM of the 40 block convolutions. With N = K = 256 it has 127 flop per
                byte, below the chip's ridge of ~312 flop/byte, so HBM bounds it: `achieved` = algorithmic bytes of one launch
                (s * 36 * (T*K + N*K + T*N)) / average launch duration, against 8 TB/s. Durations come from HIP events recorded on the
@@ -436,6 +439,9 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="positions per sub-batch (0 = library default: the whole batch)")
     ap.add_argument("--batch", type=int, default=0, help="override the configuration's batch size (experiments only; the metric is quoted at the default)")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="budget of the CPU baseline leg (0 disables it)")
+    ap.add_argument("--streams", type=int, default=2, choices=[1, 2],
+                    help="2: also time the batch as two halves on two streams and report the faster way as `value` (the roofline figures always "
+                         "come from the single-stream pass, where launches do not overlap)")
     ap.add_argument("--unfused", action="store_true", help="run every layer as the reference's three calls (no cross-layer transform fusion)")
     ap.add_argument("--layer-launch", action="store_true", help="experimental: product and both transforms of a layer as one launch (slower)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -486,6 +492,37 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = 1e3 * elapsed / args.steps
     value = batch / (elapsed / args.steps)
+    execution = "the whole batch on one stream"
+    single_stream = {"value": value, "ms_per_step": ms_per_step}
+
+    # the same batch as two halves on two contexts (two streams of the one device): one half's launch starts up and drains while the
+    # other's is in its steady state. Same results bit for bit; whichever of the two ways is faster is the throughput of the step.
+    two_streams = None
+    if args.streams == 2 and batch % 2 == 0 and not args.unfused and net.chunk == batch:
+        half = batch // 2
+        contexts = [ml.Context(0), ml.Context(0)]
+        halves = [ResNet(c, half, board, planes, channels, blocks, dtype, params, to_storage, fused=True) for c in contexts]
+        for i, part in enumerate(halves):
+            part.setInput(to_storage(x[i * half:(i + 1) * half]))
+
+        def both():
+            for part in halves:
+                part.forward()
+
+        for _ in range(args.warmup):
+            both()
+        for c in contexts:
+            c.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            both()
+        for c in contexts:
+            c.synchronize()
+        t2 = (time.perf_counter() - t0) / args.steps
+        two_streams = {"value": batch / t2, "ms_per_step": 1e3 * t2}
+        if two_streams["value"] > value:
+            value, ms_per_step, execution = two_streams["value"], two_streams["ms_per_step"], "two halves of the batch on two streams"
+        del halves
 
     # instrumented run: HIP events around every launch, on the stream the kernels run on
     timer = ml.KernelTimer(ctx)
@@ -544,8 +581,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16" if dtype == "float16" else "f32",
         "data": "synthetic (Bernoulli(0.3) input planes, He-normal weights, N(0,0.01) biases, seed %d)" % seed,
         "config": {"workload": args.config, "batch": batch, "board": board, "channels": channels, "blocks": blocks,
-                   "positions_per_launch": net.chunk, "cross_layer_transform_fusion": not args.unfused},
-        "tflops_executed": net.flops_per_forward() / (elapsed / args.steps) / 1e12,
+                   "positions_per_launch": net.chunk, "cross_layer_transform_fusion": not args.unfused, "execution": execution},
+        "single_stream": single_stream, "two_streams": two_streams,
+        "tflops_executed": net.flops_per_forward() / (ms_per_step * 1e-3) / 1e12,
         "roofline": roofline,
         "gemm_mfma": {"achieved": gemm_tflops, "peak": PEAK_MFMA_TFLOPS[dtype], "unit": "TFLOP/s", "frac": gemm_tflops / PEAK_MFMA_TFLOPS[dtype],
                       "flops_per_launch": gemm_flops,

@@ -174,14 +174,21 @@ namespace
 	 * one matrix position per step, two steps in flight, and does nothing else (no MFMA, no LDS read, no store): its duration is a
 	 * lower bound for that design. v = [36][tiles][512 bytes], u = [36][columns][512 bytes].
 	 */
-	template<int T, int N>
+	/*
+	 * FROM_X: the variant in which the workgroup would make its A operand itself, by running the input transform on the pixels of its T
+	 * tiles (T / 16 images of 15 x 15 x 256 halfs = T * 7200 bytes per task, fetched here in 36 equal portions, one per step, from x =
+	 * [images][225][512 bytes]) instead of fetching their 36 x T transformed rows; the weight slice is fetched as before.
+	 */
+	template<int T, int N, bool FROM_X>
 	__global__ __launch_bounds__(512) void kernel_fused_layer_operand_stream(const uint8_t *v, const uint8_t *u, int tiles, int columns, int tasks)
 	{
 		extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
-		constexpr int A_BLOCKS = T * 512 / 1024, B_BLOCKS = N * 512 / 1024; /* 1 KB per wavefront instruction */
-		constexpr int STEP_BYTES = (A_BLOCKS + B_BLOCKS) * 1024;
-		constexpr int LOADS = (A_BLOCKS + B_BLOCKS) / 8;
-		static_assert((A_BLOCKS + B_BLOCKS) % 8 == 0, "blocks must divide over 8 wavefronts");
+		constexpr int PATCH_BYTES = T * 7200;
+		constexpr int A_BLOCKS = FROM_X ? (PATCH_BYTES / 36 + 1023) / 1024 : T * 512 / 1024; /* 1 KB per wavefront instruction */
+		constexpr int B_BLOCKS = N * 512 / 1024;
+		constexpr int BLOCKS = A_BLOCKS + B_BLOCKS;
+		constexpr int STEP_BYTES = BLOCKS * 1024;
+		constexpr int LOADS = (BLOCKS + 7) / 8;
 		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 		const int slices = columns / N;
 		for (int task = blockIdx.x; task < tasks; task += gridDim.x)
@@ -190,16 +197,24 @@ namespace
 			for (int p = 0; p < 36; p++)
 			{
 				uint8_t *buffer = lds + (p & 1) * STEP_BYTES;
-				const uint8_t *a = v + (static_cast<size_t>(p) * tiles + static_cast<size_t>(group) * T) * 512;
+				const uint8_t *a = FROM_X ? v + static_cast<size_t>(group) * PATCH_BYTES + static_cast<size_t>(p) * (A_BLOCKS * 1024)
+						: v + (static_cast<size_t>(p) * tiles + static_cast<size_t>(group) * T) * 512;
+				const uint8_t *a_last = v + static_cast<size_t>(group + 1) * PATCH_BYTES - 1024; /* FROM_X: the last portion ends with the patch */
 				const uint8_t *b = u + (static_cast<size_t>(p) * columns + static_cast<size_t>(slice) * N) * 512;
 #pragma unroll
 				for (int l = 0; l < LOADS; l++)
 				{
 					const int block = wave + 8 * l;
-					const uint8_t *src = (block < A_BLOCKS) ? a + block * 1024 : b + (block - A_BLOCKS) * 1024;
-					__builtin_amdgcn_global_load_lds((global_ptr_t) (src + lane * 16), (lds_ptr_t) (buffer + block * 1024), 16, 0, 0);
+					if (block < BLOCKS)
+					{
+						const uint8_t *src = (block < A_BLOCKS) ? a + block * 1024 : b + (block - A_BLOCKS) * 1024;
+						if (FROM_X && block < A_BLOCKS && src > a_last)
+							src = a_last;
+						__builtin_amdgcn_global_load_lds((global_ptr_t) (src + lane * 16), (lds_ptr_t) (buffer + block * 1024), 16, 0, 0);
+					}
 				}
-				/* the previous step's loads have landed in every wavefront before its buffer is overwritten by the next step */
+				/* the previous step's loads have landed in every wavefront before its buffer is overwritten by the next step (a wavefront
+				 * whose last block index falls beyond BLOCKS has one load less in flight: its wait is merely earlier than needed) */
 				__builtin_amdgcn_s_waitcnt(0x0f70 | (LOADS & 15) | ((LOADS >> 4) << 14));
 				__builtin_amdgcn_s_barrier();
 			}
@@ -233,31 +248,38 @@ namespace
 
 extern "C"
 {
-	/* v: 36 * tiles * 512 bytes, u: 36 * columns * 512 bytes; tile_group x column_slice is 32 x 64 or 64 x 32; returns the bytes one launch moves */
-	static size_t fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups)
+	/* v: 36 * tiles * 512 bytes (from_x: the pixels instead, tiles / 16 * 115200 bytes), u: 36 * columns * 512 bytes; tile_group x column_slice is
+	 * 32 x 64 or 64 x 32; returns the bytes one launch moves into LDS */
+	static size_t fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups,
+			int from_x)
 	{
 		if (tiles <= 0 || columns <= 0 || tiles % tile_group != 0 || columns % column_slice != 0 || workgroups <= 0)
 			throw std::logic_error("ceilings: ceil_fused_layer_operand_stream: bad arguments");
 		hipStream_t s = reinterpret_cast<hipStream_t>(stream);
 		const int tasks = (tiles / tile_group) * (columns / column_slice);
-		const size_t lds_bytes = 2 * static_cast<size_t>(tile_group + column_slice) * 512;
 		const uint8_t *pv = reinterpret_cast<const uint8_t*>(v), *pu = reinterpret_cast<const uint8_t*>(u);
-		if (tile_group == 32 && column_slice == 64)
-		{
-			check(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_fused_layer_operand_stream<32, 64>), hipFuncAttributeMaxDynamicSharedMemorySize,
-					static_cast<int>(lds_bytes)), "hipFuncSetAttribute");
-			hipLaunchKernelGGL((kernel_fused_layer_operand_stream<32, 64>), dim3(workgroups), dim3(512), lds_bytes, s, pv, pu, tiles, columns, tasks);
-		}
+		const int a_blocks = from_x ? (tile_group * 7200 / 36 + 1023) / 1024 : tile_group * 512 / 1024;
+		const int blocks = a_blocks + column_slice * 512 / 1024;
+		const size_t lds_bytes = 2 * static_cast<size_t>(blocks) * 1024;
+#define CEIL_LAUNCH_OPERANDS(T, N, X) \
+		do { \
+			check(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_fused_layer_operand_stream<T, N, X>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+					static_cast<int>(lds_bytes)), "hipFuncSetAttribute"); \
+			hipLaunchKernelGGL((kernel_fused_layer_operand_stream<T, N, X>), dim3(workgroups), dim3(512), lds_bytes, s, pv, pu, tiles, columns, tasks); \
+		} while (0)
+		if (tile_group == 32 && column_slice == 64 && !from_x)
+			CEIL_LAUNCH_OPERANDS(32, 64, false);
+		else if (tile_group == 64 && column_slice == 32 && !from_x)
+			CEIL_LAUNCH_OPERANDS(64, 32, false);
+		else if (tile_group == 32 && column_slice == 64)
+			CEIL_LAUNCH_OPERANDS(32, 64, true);
 		else if (tile_group == 64 && column_slice == 32)
-		{
-			check(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel_fused_layer_operand_stream<64, 32>), hipFuncAttributeMaxDynamicSharedMemorySize,
-					static_cast<int>(lds_bytes)), "hipFuncSetAttribute");
-			hipLaunchKernelGGL((kernel_fused_layer_operand_stream<64, 32>), dim3(workgroups), dim3(512), lds_bytes, s, pv, pu, tiles, columns, tasks);
-		}
+			CEIL_LAUNCH_OPERANDS(64, 32, true);
 		else
 			throw std::logic_error("ceilings: ceil_fused_layer_operand_stream: 32 x 64 or 64 x 32 only");
+#undef CEIL_LAUNCH_OPERANDS
 		check(hipGetLastError(), "launch of kernel_fused_layer_operand_stream");
-		return static_cast<size_t>(tasks) * 36 * static_cast<size_t>(tile_group + column_slice) * 512;
+		return static_cast<size_t>(tasks) * 36 * static_cast<size_t>(blocks) * 1024;
 	}
 
 	/* mode 0 read, 1 write, 2 copy; bytes must be a multiple of 16; nt != 0 uses non-temporal accesses */
@@ -304,9 +326,9 @@ extern "C"
 	}
 	/* *bytes_moved receives the bytes one launch brings into LDS */
 	int ceil_fused_layer_operand_stream(void *stream, const void *v, const void *u, int tiles, int columns, int tile_group, int column_slice, int workgroups,
-			size_t *bytes_moved)
+			int from_x, size_t *bytes_moved)
 	{
-		return guarded([&]() { *bytes_moved = fused_layer_operand_stream(stream, v, u, tiles, columns, tile_group, column_slice, workgroups); });
+		return guarded([&]() { *bytes_moved = fused_layer_operand_stream(stream, v, u, tiles, columns, tile_group, column_slice, workgroups, from_x); });
 	}
 	int ceil_stream(void *stream, void *dst, const void *src, size_t bytes, int mode, int nt, int workgroups)
 	{

@@ -343,7 +343,7 @@ class Bench:
         lib = Checked(ceil_stream=[vp, vp, vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int],
                       ceil_mfma=[vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int],
                       ceil_fused_layer_operand_stream=[vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-                                                       ctypes.POINTER(ctypes.c_size_t)])
+                                                       ctypes.c_int, ctypes.POINTER(ctypes.c_size_t)])
         stream = ctx.stream()
         mib = 1 << 20
 
@@ -403,10 +403,12 @@ class Bench:
         u = ml.Tensor((36 * columns * 512,), "uint8")
         v.zeroall(ctx)
         u.zeroall(ctx)
-        for group, width in ((32, 64), (64, 32)):
-            moved = ctypes.c_size_t(0)
-            t = self.time(lambda: lib.ceil_fused_layer_operand_stream(stream, v.ptr, u.ptr, tiles, columns, group, width, 256, ctypes.byref(moved)))
-            report("one-kernel Winograd layer: operands", "%d tiles x %d columns x 36 per task" % (group, width), t, moved.value)
+        for from_x in (0, 1):  # A operand fetched as transformed rows, or as the pixels a workgroup would transform itself
+            for group, width in ((32, 64), (64, 32)):
+                moved = ctypes.c_size_t(0)
+                t = self.time(lambda: lib.ceil_fused_layer_operand_stream(stream, v.ptr, u.ptr, tiles, columns, group, width, 256, from_x, ctypes.byref(moved)))
+                report("one-kernel Winograd layer: operands" + (", A from pixels" if from_x else ""),
+                       "%d tiles x %d columns x 36 per task" % (group, width), t, moved.value)
         v.free()
         u.free()
         out8 = ml.Tensor((4096,), "uint8")
