@@ -426,10 +426,3 @@ MLHIP_ALSO_AS_CUDA(gemm_v2)
 MLHIP_ALSO_AS_CUDA(gemm_batched_v2)
 MLHIP_ALSO_AS_CUDA(gemm_ex)
 
-#ifdef EXP_GEMM_STAMPS
-extern "C" void hip_exp_read_gemm_stamps(void *dst, size_t bytes)
-{
-	(void) hipDeviceSynchronize();
-	(void) hipMemcpyFromSymbol(dst, HIP_SYMBOL(mlhip::exp_gemm_stamps), bytes);
-}
-#endif

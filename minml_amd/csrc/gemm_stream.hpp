@@ -51,12 +51,6 @@ namespace mlhip
 		asm volatile("" ::: "memory");
 	}
 
-#ifdef EXP_GEMM_STAMPS
-	static __device__ uint64_t exp_gemm_stamps[512 * 64];
-#define EXP_GSTAMP(slot) do { if (threadIdx.x == 0 && (slot) < 64) exp_gemm_stamps[blockIdx.x * 64 + (slot)] = wall_clock64(); } while (0)
-#else
-#define EXP_GSTAMP(slot) do { } while (0)
-#endif
 	struct StreamGemmConfig
 	{
 			static constexpr int BM = 128; /* rows of A per unit */
@@ -145,7 +139,6 @@ namespace mlhip
 
 		const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
 		const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
-		EXP_GSTAMP(0);
 		int group, n_tile;
 		if (gridDim.x % (8 * n_tiles) == 0)
 		{ /* ids congruent mod 8 share an XCD: give the column slices of one group consecutive slots of one XCD */
@@ -412,14 +405,12 @@ namespace mlhip
 			for (int g = 0; g < DISTANCE; g++)
 				if (g < run_stages)
 					request_stage(g);
-			EXP_GSTAMP(1);
 			/* Loads return in order: once at most the stages requested after stage 0 are outstanding, the B operand (requested first) and
 			 * stage 0 have landed, and the first k steps run while the rest of the ring is still filling (no change where HBM bounds the
 			 * launch; 59 -> 57 us for the fp32 products of 4096 tiles at 128 channels). The explicit wait also tells the compiler that no
 			 * register load is outstanding any more, so it guards nothing inside the loop. */
 			wait_vmcnt_stages<LOADS>(min(DISTANCE, run_stages) - 1);
 			barrier_no_fence();
-			EXP_GSTAMP(2);
 			clear_accumulators();
 			read_fragments(0, 0, frags[0]);
 
@@ -465,9 +456,7 @@ namespace mlhip
 						Traits::mma(b_regs[t], frags[cur][i], acc[i]);
 					__builtin_amdgcn_sched_barrier(0);
 				});
-				EXP_GSTAMP(4 + 2 * u);
 				store_unit(u);
-				EXP_GSTAMP(5 + 2 * u);
 				clear_accumulators();
 			};
 			/* steady while the last stage of the unit can still request DISTANCE stages ahead */
@@ -479,10 +468,6 @@ namespace mlhip
 				process_unit(u, std::false_type());
 			unit = run_end;
 		}
-#ifdef EXP_GEMM_STAMPS
-		__builtin_amdgcn_s_waitcnt(0);
-		EXP_GSTAMP(3);
-#endif
 	}
 	/* operands of one streaming launch: `batch` products C[i] = A[i] * B[i]^T with K rows of k_bytes bytes (strides in elements) */
 	struct StreamGemmArgs

@@ -258,11 +258,8 @@ namespace
 	 * ACT: 0 = linear, 1 = ReLU (both fused as the reference fuses them), 2 = any other activation, selected at run time.
 	 * The 36 matrix rows and the 16 residual vectors (from clamped coordinates) are requested before any arithmetic.
 	 */
-#ifndef EXP_OUT_BLOCKS
-#define EXP_OUT_BLOCKS 1
-#endif
 	template<typename T, int VEC, int ACT, bool HAS_EXT>
-	__global__ __launch_bounds__(256, EXP_OUT_BLOCKS) void kernel_output_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+	__global__ __launch_bounds__(256) void kernel_output_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
 			const T *ext, int act, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
 	{
 		typedef typename RawVec<T, VEC>::type raw_t;
@@ -371,12 +368,6 @@ namespace
 		}
 	}
 
-#ifdef EXP_TIMESTAMPS
-	__device__ uint64_t exp_stamps[8192 * 8];
-#define EXP_STAMP(slot) do { if (threadIdx.x == 0) exp_stamps[blockIdx.x * 8 + (slot)] = wall_clock64(); } while (0)
-#else
-#define EXP_STAMP(slot) do { } while (0)
-#endif
 	/* one image's share of a fused output -> input transform: where its matrices, pixels and next matrices lie */
 	template<typename T>
 	struct FusedImage
@@ -480,11 +471,6 @@ namespace
 			if (!loaded)
 				load_matrices(in_image);
 			loaded = false;
-#ifdef EXP_TIMESTAMPS
-			EXP_STAMP(1);
-			__builtin_amdgcn_s_waitcnt(0x0f70); /* vmcnt(0) */
-			EXP_STAMP(2);
-#endif
 			const int tile_x = in_image / tiles_w;
 			const int x0 = 4 * tile_x;
 			const int y0 = 4 * (in_image - tile_x * tiles_w);
@@ -652,10 +638,7 @@ namespace
 	 * the write and re-read of y through HBM (or only the re-read, when y is also needed as a later residual).
 	 */
 	template<typename T, int VEC, int SLICE, int ACT, bool HAS_EXT, int THREADS>
-	#ifndef EXP_FUSED_THREADS_PER_CU
-#define EXP_FUSED_THREADS_PER_CU 512
-#endif
-	__global__ __launch_bounds__(THREADS, ((VEC <= 2) ? 1024 : EXP_FUSED_THREADS_PER_CU) / THREADS) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
+		__global__ __launch_bounds__(THREADS, ((VEC <= 2) ? 1024 : 512) / THREADS) void kernel_output_input_transform_4x4_3x3(const T *__restrict__ matrices, T *output, const T *__restrict__ bias,
 			const T *ext, int act, T *__restrict__ next_matrices, int batch_size, int height, int width, int channels, int tiles_h, int tiles_w)
 	{
 		extern __shared__ __attribute__((aligned(16))) uint8_t lds_bytes[];
@@ -688,25 +671,9 @@ namespace
 		 * is touched once here), the next layer's matrices are written cacheable, because the product that follows walks them from
 		 * the end and finds the rows written last still in the last-level cache.
 		 */
-		EXP_STAMP(0);
 		fused_transform_phase1<T, VEC, SLICE, ACT, HAS_EXT, THREADS, true, true>(g, lds_bytes);
-		EXP_STAMP(3);
 		__syncthreads();
-		EXP_STAMP(4);
 		fused_transform_phase2<T, VEC, SLICE, THREADS, false>(g, lds_bytes);
-		EXP_STAMP(6);
-#ifdef EXP_TIMESTAMPS
-		__builtin_amdgcn_s_waitcnt(0); /* all stores acknowledged */
-		EXP_STAMP(7);
-		if (threadIdx.x == 0)
-		{
-			unsigned int xcc;
-			asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-			unsigned int hwid;
-			asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-			exp_stamps[blockIdx.x * 8 + 5] = (static_cast<uint64_t>(xcc & 15) << 32) | hwid;
-		}
-#endif
 	}
 
 	/* ---------------------------------------------------------------------------------------------------------------------
@@ -1233,14 +1200,6 @@ namespace mlhip
 		(void) layer_static_pointer(device_index);
 	}
 }
-
-#ifdef EXP_TIMESTAMPS
-extern "C" void hip_exp_read_stamps(void *dst, size_t bytes)
-{
-	(void) hipDeviceSynchronize();
-	(void) hipMemcpyFromSymbol(dst, HIP_SYMBOL(exp_stamps), bytes);
-}
-#endif
 
 extern "C"
 {
