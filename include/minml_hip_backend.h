@@ -152,6 +152,11 @@ extern "C"
 	/* ---- GEMMs (reference: cuda_backend.h:147-154; semantics of src/backend/cpu/gemm/gemm.cpp:34-83).
 	 *      C.dtype == INT32 selects the int8 x int8 -> int32 product (src/backend/cuda/gemms.cpp:119-130). ---- */
 	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C);
+	/* grouped product (reference: cuda_backend.h:239-240, src/backend/cuda/kernels/group_conv.cu:120-203; reached from the grouped 1x1
+	 * convolution, src/layers/Conv2D.cpp:341-349 via src/core/math.cpp:1079-1093): the last dimension of A, B and C is split into `groups`
+	 * equal column ranges and group i computes C[:, i-th range] = alpha * op(A[:, i-th range]) * op(B[:, i-th range]) + beta * C[:, i-th range].
+	 * The reference has no CPU implementation of it; it is checked against the definition (one plain product per group). */
+	void hip_group_gemm(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C, int groups);
 	void hip_gemm_batched_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C);
 	void hip_gemm(mlContext_t context, mlDataType_t dtype, mlShape_t shape_C, void *C, mlShape_t shape_A, const void *A, mlShape_t shape_B,
 			const void *B, char opA, char opB, float alpha, float beta);

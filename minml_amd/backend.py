@@ -98,6 +98,7 @@ SIGNATURES = {
     "activation_forward": (None, [_vp, _f, _T, _f, _T, _i]),
     "add_tensors": (None, [_vp, _f, _T, _f, _T, _f, _T, _f, _T]),
     "scale_tensor": (None, [_vp, _f, _T]),
+    "group_gemm": (None, [_vp, _c, _c, _f, _T, _T, _f, _T, _i]),
     "softmax_forward": (None, [_vp, _i, _S, _vp, _vp]),
     "global_average_pooling_forward": (None, [_vp, _f, _T, _f, _T]),
     "batchnorm_inference": (None, [_vp, _f, _T, _T, _T, _T, _f, _T, _i]),

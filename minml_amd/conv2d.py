@@ -7,6 +7,8 @@ What is mirrored, with the reference lines it follows:
   * Winograd sequence: input transform into workspace[0 : 36*T*Cin], gemmBatched('n','t'), output transform from
     workspace[36*T*Cin : ...] with bias / residual / activation       Conv2D.cpp:365-378
   * explicit GEMM (1x1)                                     Conv2D.cpp:329-353 -> src/core/math.cpp:1595-1626
+  * grouped convolution (groups > 1): grouped product on the flattened tensors, then bias + activation as a second call
+                                                            Conv2D.cpp:71-101 (weights [Cout / groups, k, k, Cin]), :339-349
   * int8 path: im2row with zero-point padding -> int8 GEMM -> quantized_scale_shift_act      Conv2D.cpp:214-239
   * quantisation set-up                                     src/layers/Layer.cpp:147-160, src/layers/quantization.cpp:55-93
 
@@ -35,14 +37,18 @@ def get_weight_matrices_shape(weight_shape, tile_size):
 
 
 class Conv2D:
-    def __init__(self, context, input_shape, filters, kernel_size, activation="linear", use_bias=True, dtype="float16", algorithm=None):
+    def __init__(self, context, input_shape, filters, kernel_size, activation="linear", use_bias=True, dtype="float16", algorithm=None, groups=1):
         self.context = context
+        self.groups = groups
+        if groups != 1 and (input_shape[3] % groups != 0 or filters % groups != 0 or kernel_size != 1):
+            # the reference flattens input and weights to matrices (Conv2D.cpp:341-344), which is a convolution only for a 1x1 kernel
+            raise ValueError("grouped convolution: 1x1 kernels, filters divisible by the number of groups")
         self.input_shape = tuple(input_shape)
         self.kernel_size = kernel_size
         self.activation = ml.act_of(activation)
         self.use_bias = use_bias
         self.dtype = ml.dtype_of(dtype)
-        self.weight_shape = (filters, kernel_size, kernel_size, input_shape[3])
+        self.weight_shape = (filters // groups, kernel_size, kernel_size, input_shape[3])
         self.output_shape = (input_shape[0], input_shape[1], input_shape[2], filters)
         self.weights = None
         self.bias = None
@@ -116,6 +122,16 @@ class Conv2D:
 
         if self.forward_algorithm == IMPLICIT_GEMM:
             ml.convolutionImplicitGemmForward(ctx, x, self.weights, output, self.bias, add, self.activation)
+        elif self.forward_algorithm == EXPLICIT_GEMM and self.groups > 1:
+            if add is not None:
+                raise ValueError("a grouped convolution takes no second input")
+            rows = x.volume() // x.lastDim()
+            output_matrix = output.view((rows, output.lastDim()))
+            ml.gemmGrouped(ctx, "n", "t", output_matrix, x.view((rows, x.lastDim())), self.weights.view((self.weights.firstDim(), self.weights.volume() // self.weights.firstDim())), 1.0, 0.0, self.groups)
+            if self.bias is not None:
+                ml.addBiasAct(ctx, 1.0, output, self.bias, 0.0, output, self.activation)
+            else:
+                ml.activationForward(ctx, 1.0, output, 0.0, output, self.activation)
         elif self.forward_algorithm == EXPLICIT_GEMM:
             ml.explicit_gemm_forward(ctx, x, output, self.weights, self.bias, workspace, self.activation, add)
         else:

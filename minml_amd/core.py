@@ -446,6 +446,21 @@ def gemm(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
     _launch("gemm_v2", context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc())
 
 
+def gemmGrouped(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0, groups=1):
+    """The last dimension of A, B and C is cut into `groups` equal column ranges; range i of C = alpha op(A range i) op(B range i) + beta C
+    (reference: src/core/math.cpp:1079-1093, device only; shapes as src/backend/cuda/kernels/group_conv.cu:120-139 derives them)."""
+    _require(A.rank() == 2 and Bm.rank() == 2 and C.rank() == 2, "gemmGrouped takes matrices")
+    _require(groups >= 1 and A.shape[1] % groups == 0 and Bm.shape[1] % groups == 0 and C.shape[1] % groups == 0, "last dimensions must be multiples of groups")
+    _require(opA in "ntNT" and opB in "ntNT", "op must be n or t")
+    ta, tb = opA in "tT", opB in "tT"
+    M = A.shape[1] // groups if ta else A.shape[0]
+    K = A.shape[0] if ta else A.shape[1] // groups
+    N = Bm.shape[0] if tb else Bm.shape[1] // groups
+    _require((Bm.shape[1] // groups if tb else Bm.shape[0]) == K and C.shape == (M, N * groups), "shapes do not agree")
+    _require(_same_dtype(A, Bm, C) and C.dtype in (B.DTYPE_FLOAT16, B.DTYPE_FLOAT32), "dtype mismatch")
+    _launch("group_gemm", context.handle, opA.encode(), opB.encode(), alpha, A.desc(), Bm.desc(), beta, C.desc(), groups)
+
+
 def gemmBatched(context, opA, opB, C, A, Bm, alpha=1.0, beta=0.0):
     """reference: src/core/math.cpp:662-680; rank-2 operands are broadcast over the batch."""
     _require(C.rank() == 3 and (A.rank() == 3 or Bm.rank() == 3), "gemmBatched takes rank-3 tensors")

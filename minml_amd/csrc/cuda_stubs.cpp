@@ -60,7 +60,6 @@ MLHIP_STUB(cuda_layernorm_backward)
 MLHIP_STUB(cuda_rmsnorm_backward)
 /* attention, mixture of experts */
 MLHIP_STUB(cuda_multi_head_attention_backward)
-MLHIP_STUB(cuda_group_gemm)
 MLHIP_STUB(cuda_token_choice_routing_backward)
 MLHIP_STUB(cuda_expert_choice_routing_backward)
 MLHIP_STUB(cuda_select_top_k)

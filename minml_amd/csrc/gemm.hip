@@ -48,7 +48,7 @@ namespace
 	/* Fallback: one thread per output element, any op combination, any alignment. */
 	template<typename T, typename AccT, typename Epilogue>
 	__global__ __launch_bounds__(256) void kernel_gemm_generic(const T *A, const T *B, int M, int N, int K, size_t a_row, size_t a_col, size_t b_row,
-			size_t b_col, size_t stride_a, size_t stride_b, size_t stride_c, Epilogue epilogue)
+			size_t b_col, size_t stride_a, size_t stride_b, size_t stride_c, Epilogue epilogue, int out_stride)
 	{
 		const size_t gid = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
 		if (gid >= static_cast<size_t>(M) * N)
@@ -75,7 +75,7 @@ namespace
 		Epilogue single = local;
 		const AccT vals[4] = { acc, 0, 0, 0 };
 		single.N = n + 1;
-		single.row_stride = N;
+		single.row_stride = out_stride; /* elements between consecutive rows of D and C */
 		single(m, n, vals);
 	}
 
@@ -98,6 +98,99 @@ namespace
 		ep.act = g.act;
 		ep.vectorized = vectorized;
 		return ep;
+	}
+	/*
+	 * Tall products with very few columns (the 1x1 policy head: [B*H*W, C] x [1, C]^T): a matrix-vector product per column, bound by the
+	 * read of A. One row of A is 16 bytes per lane on LANES lanes (K rows of 16 ... 1024 bytes, LANES a power of two), so a wavefront
+	 * instruction covers 64 / LANES consecutive rows = 1 KB of consecutive memory; the lanes of a row hold their 16-byte pieces of the
+	 * NMAX rows of B in registers, multiply, and meet in a butterfly of cross-lane additions; the row's first lane applies the epilogue.
+	 * Four row groups are in flight per wavefront.
+	 */
+	template<typename T, int NMAX>
+	__global__ __launch_bounds__(256) void kernel_gemv_rows(const T *A, const T *B, int M, int N, int lanes, size_t k_elements, FloatEpilogue<T> epilogue)
+	{
+		constexpr int E = 16 / sizeof(T); /* elements per 16-byte piece */
+		constexpr int UNROLL = 4;
+		const int lane = threadIdx.x & 63;
+		const int piece = lane & (lanes - 1), row_in_group = lane / lanes;
+		const int rows_per_group = 64 / lanes;
+		float b[NMAX][E];
+#pragma unroll
+		for (int n = 0; n < NMAX; n++)
+		{
+			Vec<T, E> tmp;
+			if (n < N)
+				tmp.load(B + static_cast<size_t>(n) * k_elements + piece * E);
+			else
+				tmp.zero();
+#pragma unroll
+			for (int e = 0; e < E; e++)
+				b[n][e] = tmp.v[e];
+		}
+		epilogue.vectorized = false;
+		const size_t wave = (static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x) >> 6;
+		const size_t waves = (static_cast<size_t>(gridDim.x) * blockDim.x) >> 6;
+		const size_t groups = (static_cast<size_t>(M) + rows_per_group - 1) / rows_per_group;
+		for (size_t first = wave * UNROLL; first < groups; first += waves * UNROLL)
+		{
+			Vec<T, E> a[UNROLL];
+#pragma unroll
+			for (int u = 0; u < UNROLL; u++)
+			{
+				const size_t m = min((first + u) * rows_per_group + row_in_group, static_cast<size_t>(M) - 1);
+				a[u].load(A + m * k_elements + piece * E);
+			}
+#pragma unroll
+			for (int u = 0; u < UNROLL; u++)
+			{
+				float sum[NMAX];
+#pragma unroll
+				for (int n = 0; n < NMAX; n++)
+				{
+					sum[n] = 0.0f;
+#pragma unroll
+					for (int e = 0; e < E; e++)
+						sum[n] = fmaf(a[u].v[e], b[n][e], sum[n]);
+				}
+				for (int offset = 1; offset < lanes; offset <<= 1)
+#pragma unroll
+					for (int n = 0; n < NMAX; n++)
+						sum[n] += __shfl_xor(sum[n], offset);
+				const size_t m = (first + u) * rows_per_group + row_in_group;
+				if (piece == 0 && first + u < groups && m < static_cast<size_t>(M))
+				{
+#pragma unroll
+					for (int n = 0; n < NMAX; n++)
+						if (n < N)
+						{
+							FloatEpilogue<T> single = epilogue;
+							const float vals[4] = { sum[n], 0.0f, 0.0f, 0.0f };
+							single.N = n + 1; /* the other members of the group of 4 lie outside the matrix */
+							single(static_cast<int>(m), n, vals);
+						}
+				}
+			}
+		}
+	}
+	template<typename T>
+	bool try_launch_gemv(hipStream_t stream, const GemmArgs &g, bool fast, size_t k_bytes)
+	{
+		const size_t pieces = k_bytes / 16;
+		if (!(fast && g.batch == 1 && g.N >= 1 && g.N <= 4 && k_bytes % 16 == 0 && pieces >= 1 && pieces <= 64 && (pieces & (pieces - 1)) == 0))
+			return false;
+		FloatEpilogue<T> ep = make_float_epilogue<T>(g, false);
+		const int rows_per_group = 64 / static_cast<int>(pieces);
+		const size_t groups = (static_cast<size_t>(g.M) + rows_per_group - 1) / rows_per_group;
+		/* 4 wavefronts per workgroup, 4 row groups per wavefront and round; enough workgroups for 8 wavefronts per SIMD */
+		const size_t wanted = (groups + 15) / 16;
+		const unsigned int grid = static_cast<unsigned int>(std::min<size_t>(wanted, static_cast<size_t>(device_compute_units()) * 8));
+		if (g.N == 1)
+			hipLaunchKernelGGL((kernel_gemv_rows<T, 1>), dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B), g.M, g.N,
+					static_cast<int>(pieces), static_cast<size_t>(g.K), ep);
+		else
+			hipLaunchKernelGGL((kernel_gemv_rows<T, 4>), dim3(grid), dim3(256), 0, stream, reinterpret_cast<const T*>(g.A), reinterpret_cast<const T*>(g.B), g.M, g.N,
+					static_cast<int>(pieces), static_cast<size_t>(g.K), ep);
+		return true;
 	}
 }
 
@@ -136,6 +229,13 @@ namespace mlhip
 		const bool vectorized = (g.N % 4 == 0) && aligned_to(g.D, 4 * out_size) && aligned_to(g.C, 4 * out_size) && aligned_to(g.bias, 4 * esize)
 				&& ((g.stride_c * out_size) % (4 * out_size) == 0);
 
+		/* products with at most 4 columns (policy heads): one pass over A, no matrix cores; taken at every number of rows, so that a
+		 * position's result does not depend on the size of the batch it is part of */
+		if ((g.dtype == DTYPE_FLOAT16 && try_launch_gemv<half_t>(stream, g, fast, k_bytes)) || (g.dtype == DTYPE_FLOAT32 && try_launch_gemv<float>(stream, g, fast, k_bytes)))
+		{
+			MLHIP_CHECK(hipGetLastError());
+			return;
+		}
 		/*
 		 * Products with short K rows (128 / 256 / 512 bytes) and many rows are bound by HBM: they take the persistent streaming kernel -
 		 * the Winograd products with a plain 16-byte store, everything else (gemm_ex, 1x1 convolutions, the int8 product) with the
@@ -222,7 +322,7 @@ namespace mlhip
 				else
 					hipLaunchKernelGGL((kernel_gemm_generic<half_t, float, FloatEpilogue<half_t>>), slow_grid, dim3(256), 0, stream,
 							reinterpret_cast<const half_t*>(g.A), reinterpret_cast<const half_t*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
-							g.stride_b, g.stride_c, ep);
+							g.stride_b, g.stride_c, ep, g.N);
 				break;
 			}
 			case DTYPE_FLOAT32:
@@ -247,7 +347,7 @@ namespace mlhip
 				else
 					hipLaunchKernelGGL((kernel_gemm_generic<float, float, FloatEpilogue<float>>), slow_grid, dim3(256), 0, stream,
 							reinterpret_cast<const float*>(g.A), reinterpret_cast<const float*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
-							g.stride_b, g.stride_c, ep);
+							g.stride_b, g.stride_c, ep, g.N);
 				break;
 			}
 			case DTYPE_INT8:
@@ -268,7 +368,7 @@ namespace mlhip
 				else
 					hipLaunchKernelGGL((kernel_gemm_generic<int8_t, int, Int32Epilogue>), slow_grid, dim3(256), 0, stream,
 							reinterpret_cast<const int8_t*>(g.A), reinterpret_cast<const int8_t*>(g.B), g.M, g.N, g.K, a_row, a_col, b_row, b_col, g.stride_a,
-							g.stride_b, g.stride_c, ep);
+							g.stride_b, g.stride_c, ep, g.N);
 				break;
 			}
 			default:
@@ -365,6 +465,69 @@ extern "C"
 	{
 		return mlhip::entry_failed<void>();
 	}
+	void hip_group_gemm(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C, int groups)
+	try
+	{
+		MLHIP_REQUIRE(A.rank == 2 && B.rank == 2 && C.rank == 2, "group_gemm: A, B and C must be matrices");
+		MLHIP_REQUIRE(groups > 0 && A.dim[1] % groups == 0 && B.dim[1] % groups == 0 && C.dim[1] % groups == 0,
+				"group_gemm: the last dimension of every matrix must be a multiple of the number of groups");
+		MLHIP_REQUIRE(A.dtype == C.dtype && B.dtype == C.dtype && (C.dtype == DTYPE_FLOAT16 || C.dtype == DTYPE_FLOAT32), "group_gemm: fp16 or fp32 matrices of one type");
+		const bool ta = is_transpose(opA), tb = is_transpose(opB);
+		const int lda = A.dim[1], ldb = B.dim[1], ldc = C.dim[1];
+		const int part_a = lda / groups, part_b = ldb / groups, part_c = ldc / groups; /* columns of one group in each matrix */
+		const int M = ta ? part_a : A.dim[0], K = ta ? A.dim[0] : part_a, N = tb ? B.dim[0] : part_b;
+		MLHIP_REQUIRE((tb ? part_b : B.dim[0]) == K && C.dim[0] == M && part_c == N, "group_gemm: shapes do not agree");
+		if (M == 0 || N == 0)
+			return;
+		MLHIP_REQUIRE(A.data != nullptr && B.data != nullptr && C.data != nullptr && groups <= 65535, "group_gemm: null matrix or too many groups");
+		const hipStream_t stream = stream_of(context);
+		const int esize = size_of(C.dtype);
+		const size_t k_bytes = static_cast<size_t>(K) * esize;
+		const auto launch = [&](auto zero)
+		{
+			typedef decltype(zero) T;
+			FloatEpilogue<T> ep;
+			ep.D = reinterpret_cast<T*>(C.data);
+			ep.C = reinterpret_cast<const T*>(C.data);
+			ep.bias = nullptr;
+			ep.N = N;
+			ep.row_stride = ldc;
+			ep.alpha = alpha;
+			ep.beta = beta;
+			ep.act = ACTIVATION_LINEAR;
+			ep.vectorized = N % 4 == 0 && aligned_to(C.data, 4 * esize) && (static_cast<size_t>(ldc) * esize) % (4 * esize) == 0;
+			const bool dma = !ta && tb && K > 0 && k_bytes % 128 == 0 && aligned_to(A.data, 16) && aligned_to(B.data, 16)
+					&& static_cast<size_t>(lda) * esize <= 0x7fffffffu && static_cast<size_t>(ldb) * esize <= 0x7fffffffu;
+			if (dma)
+			{
+				/* the forward form of a grouped 1x1 convolution: the groups are the matrices of one launch of the tile engine, whose operand
+				 * rows may lie any distance apart; group i starts i * K elements into the rows of A and B and i * N elements into those of C */
+				DenseDmaRows a_loader { reinterpret_cast<const uint8_t*>(A.data), M, static_cast<int>(k_bytes) };
+				a_loader.row_stride_bytes = static_cast<int>(static_cast<size_t>(lda) * esize);
+				DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(B.data), N, static_cast<int>(k_bytes) };
+				b_loader.row_stride_bytes = static_cast<int>(static_cast<size_t>(ldb) * esize);
+				launch_gemm_dma<T>(stream, a_loader, b_loader, M, N, static_cast<int>(k_bytes), groups, k_bytes, k_bytes, static_cast<size_t>(N), ep);
+			}
+			else
+			{
+				const size_t a_row = ta ? 1 : lda, a_col = ta ? lda : 1, b_row = tb ? ldb : 1, b_col = tb ? 1 : ldb;
+				const size_t outputs = static_cast<size_t>(M) * N;
+				MLHIP_REQUIRE((outputs + 255) / 256 <= 0x7fffffffu, "group_gemm: too large");
+				hipLaunchKernelGGL((kernel_gemm_generic<T, float, FloatEpilogue<T>>), dim3(static_cast<unsigned int>((outputs + 255) / 256), groups), dim3(256), 0,
+						stream, reinterpret_cast<const T*>(A.data), reinterpret_cast<const T*>(B.data), M, N, K, a_row, a_col, b_row, b_col,
+						static_cast<size_t>(part_a), static_cast<size_t>(part_b), static_cast<size_t>(part_c), ep, ldc);
+			}
+		};
+		if (C.dtype == DTYPE_FLOAT16)
+			launch(half_t(0));
+		else
+			launch(0.0f);
+		MLHIP_CHECK(hipGetLastError());
+	}
+	catch (...)
+	{
+		return mlhip::entry_failed<void>();
+	}
 	void hip_gemm_v2(mlContext_t context, char opA, char opB, float alpha, const mlTensor_t A, const mlTensor_t B, float beta, mlTensor_t C)
 	try
 	{
@@ -425,4 +588,4 @@ MLHIP_ALSO_AS_CUDA(gemm_batched)
 MLHIP_ALSO_AS_CUDA(gemm_v2)
 MLHIP_ALSO_AS_CUDA(gemm_batched_v2)
 MLHIP_ALSO_AS_CUDA(gemm_ex)
-
+MLHIP_ALSO_AS_CUDA(group_gemm)

@@ -406,3 +406,79 @@ def test_convert_type_vector_body_and_tail(ctx, elements):
     back = ml.Tensor((elements,), "float32")
     ml.convertType(ctx, back, dst)
     assert np.array_equal(back.copyToHost(ctx), O.from_half(got))
+
+
+# ---- grouped product (reference: src/core/math.cpp:1079-1093, device backend only; checked against its definition) ---------------
+def _grouped_reference(opA, opB, A, Bm, C, alpha, beta, groups):
+    """One plain product of the oracle per group, on the group's column ranges."""
+    ta, tb = opA == "t", opB == "t"
+    pa, pb, pc = A.shape[1] // groups, Bm.shape[1] // groups, C.shape[1] // groups
+    out = C.copy()
+    for g in range(groups):
+        a = np.ascontiguousarray(A[:, g * pa:(g + 1) * pa])
+        b = np.ascontiguousarray(Bm[:, g * pb:(g + 1) * pb])
+        c = np.ascontiguousarray(C[:, g * pc:(g + 1) * pc])
+        out[:, g * pc:(g + 1) * pc] = O.gemm(a, b, opA, opB, alpha, beta, c if beta != 0.0 else None)
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32"])
+@pytest.mark.parametrize("case", [("n", "t", 300, 32, 64, 4, 1.0, 0.0), ("n", "t", 1000, 64, 256, 2, 1.0, 0.0), ("n", "t", 77, 12, 20, 3, 0.5, 1.5),
+                                  ("n", "t", 513, 36, 128, 8, 1.0, 1.0), ("n", "n", 45, 24, 16, 2, 1.0, 0.0), ("t", "n", 30, 28, 50, 4, 2.0, 0.0)])
+def test_group_gemm(ctx, dtype, case):
+    """K rows of whole 128-byte chunks take the tile engine with the groups as its batch (operand rows a whole matrix row apart);
+    everything else, the transposed forms of the backward pass included, the one-thread-per-output kernel."""
+    opA, opB, M, N, K, groups, alpha, beta = case
+    rng = np.random.default_rng(M + N + K)
+    a_shape = (K, M * groups) if opA == "t" else (M, K * groups)
+    b_shape = (N, K * groups) if opB == "t" else (K, N * groups)
+    A = random_tensor(rng, a_shape, dtype)
+    Bm = random_tensor(rng, b_shape, dtype, (1.0 / K) ** 0.5)
+    C0 = random_tensor(rng, (M, N * groups), dtype)
+    dC = ml.toDevice(ctx, C0)
+    ml.gemmGrouped(ctx, opA, opB, dC, ml.toDevice(ctx, A), ml.toDevice(ctx, Bm), alpha, beta, groups)
+    want = _grouped_reference(opA, opB, A, Bm, C0, alpha, beta, groups)
+    assert max_abs_rel(dC.copyToHost(ctx), want) <= TOL[dtype]
+
+
+def test_grouped_1x1_convolution_layer(ctx):
+    """Conv2D with groups > 1 as the reference runs it (src/layers/Conv2D.cpp:339-349): grouped product, then bias and activation; against
+    one dense 1x1 convolution of the oracle per group."""
+    from minml_amd.conv2d import Conv2D
+
+    rng = np.random.default_rng(5)
+    batch, board, cin, cout, groups = 3, 9, 128, 96, 4
+    x = random_tensor(rng, (batch, board, board, cin), "float16")
+    w = random_tensor(rng, (cout // groups, 1, 1, cin), "float16", 0.2)
+    b = random_tensor(rng, (cout,), "float16", 0.1)
+    layer = Conv2D(ctx, x.shape, cout, 1, "relu", True, "float16", groups=groups)
+    layer.setWeights(w, b)
+    y = ml.Tensor((batch, board, board, cout), "float16")
+    layer.forward([ml.toDevice(ctx, x)], y)
+    want = np.zeros((batch, board, board, cout), np.uint16)
+    ci, co = cin // groups, cout // groups
+    for g in range(groups):
+        wg = np.ascontiguousarray(w[:, :, :, g * ci:(g + 1) * ci])
+        # the reference stores the product, then adds bias and applies the activation in a second call: two roundings to fp16
+        product = O.conv2d_forward(np.ascontiguousarray(x[..., g * ci:(g + 1) * ci]), wg, None, None, O.LINEAR)
+        want[..., g * co:(g + 1) * co] = O.add_bias_act(product, np.ascontiguousarray(b[g * co:(g + 1) * co]), O.RELU)
+    assert max_abs_rel(y.copyToHost(ctx), want) <= 1e-2
+
+
+@pytest.mark.parametrize("dtype", ["float16", "float32"])
+@pytest.mark.parametrize("case", [(230400 // 8, 1, 256), (5000, 1, 128), (4100, 3, 64), (4097, 4, 32), (6000, 2, 8), (4096, 1, 24), (9001, 1, 512), (7, 1, 256), (225, 2, 128)])
+def test_gemm_ex_tall_with_few_columns(ctx, dtype, case):
+    """Policy-head shapes: 1 to 4 columns, few to many rows. K rows of 16 * 2^i bytes take the one-pass matrix-vector kernel (every
+    row block size from 1 to 64 lanes per row, ragged last groups); 24 elements per row take the general route. Bias, beta and ReLU included."""
+    M, N, K = case
+    rng = np.random.default_rng(M + N + K)
+    A = random_tensor(rng, (M, K), dtype)
+    Bm = random_tensor(rng, (N, K), dtype, (1.0 / K) ** 0.5)
+    bias = random_tensor(rng, (N,), dtype, 0.3)
+    C = random_tensor(rng, (M, N), dtype)
+    dA, dB = ml.toDevice(ctx, A), ml.toDevice(ctx, Bm)
+    dD = ml.Tensor((M, N), dtype)
+    ml.gemm_ex(ctx, dD, 1.0, "n", dA, "t", dB, 0.0, None, ml.toDevice(ctx, bias), "linear")
+    assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, bias=bias, act=O.LINEAR)) <= TOL[dtype]
+    ml.gemm_ex(ctx, dD, 1.25, "n", dA, "t", dB, 0.5, ml.toDevice(ctx, C), ml.toDevice(ctx, bias), "relu")
+    assert max_abs_rel(dD.copyToHost(ctx), O.gemm(A, Bm, alpha=1.25, beta=0.5, C=C, bias=bias, act=O.RELU)) <= TOL[dtype]

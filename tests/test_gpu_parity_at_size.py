@@ -118,3 +118,34 @@ def test_config5_33_positions_at_batch_256(ctx, moe):
           % ("with experts" if moe else "attention halves only", len(sample), sample[0], sample[-1], {k: "%.2e" % v for k, v in sorted(worst.items())}),
           flush=True)
     assert max(worst.values()) <= 1e-2, worst
+
+
+def test_config3_every_layer_of_33_positions_at_batch_1024_bit_exact(ctx):
+    """Config 3 as benchmarked (the int8 form of config 2, activation ranges calibrated on 64 batches, B = 1024): the int8 output of all
+    41 3x3 layers and the fp32 head of positions 0, 32, ..., 992 and 1023, bit for bit against the oracle's restatement of the
+    reference's integer branch (src/layers/Conv2D.cpp:240-308; itself held to vectors recorded from the reference's own layer,
+    tests/test_oracle_int8_reference.py)."""
+    from minml_amd import quantization as Q
+    from minml_amd.resnet import QuantizedResNet, calibrate_activations
+    from oracle.cpu_net import CpuQuantizedResNet
+
+    O.set_num_threads(16)
+    board, planes, channels, blocks, batch = 15, 32, 256, 20, 1024
+    sample = spread(batch, 32)
+    params = make_parameters(1, planes, channels, blocks)
+    ranges = calibrate_activations(ctx, params, board, planes, channels, blocks, batches=64, batch_size=4, seed=1)
+    x = make_input(1, batch, board, planes)
+    net = QuantizedResNet(ctx, batch, board, planes, channels, blocks, params, ranges)
+    seen = {}
+    net.observer = lambda index, tensor: seen.__setitem__(index, tensor.copyToHost(ctx)[sample])
+    net.setInput(x)
+    head = net.forward().copyToHost(ctx)
+    want_layers = []
+    want_head = CpuQuantizedResNet(net.host_parameters, blocks).forward(Q.quantize_tensor(x[sample], net.transforms[0]), want_layers)
+    assert len(want_layers) == 1 + 2 * blocks == len(seen)
+    wrong = [mismatches(seen[i], want_layers[i]) for i in range(len(want_layers))]
+    print("config 3, batch 1024, int8, %d positions (%d ... %d): mismatching int8 outputs per 3x3 layer: %s; mismatching fp32 logits: %d"
+          % (len(sample), sample[0], sample[-1], wrong, mismatches(head[sample], want_head)), flush=True)
+    assert not any(wrong)
+    assert np.array_equal(head[sample], want_head)
+    assert max(int(np.abs(seen[i].astype(np.int32)).max()) for i in seen) > 20  # the calibrated ranges are in use
