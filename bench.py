@@ -219,7 +219,7 @@ def run_int8(args, ml):
                      + " (3x3 convolution as implicit GEMM, M=%d N=%d K=%d)" % (pix, channels, 9 * channels),
                      "algorithmic_ops": conv_ops, "algorithmic_bytes": conv_bytes, "launches_timed": count, "avg_launch_us": t_conv * 1e6},
     }
-    if not args.unfused:
+    if not args.unfused and not args.skip_three_call:
         # the reference's route for an int8 layer on a device: im2row -> int8 GEMM into int32 -> requantisation (src/layers/Conv2D.cpp:214-239)
         three = QuantizedResNet(ctx, batch, board, planes, channels, blocks, params, ranges, "reference")
         three.setInput(x)
@@ -442,6 +442,8 @@ def main():
     ap.add_argument("--streams", type=int, default=2, choices=[1, 2],
                     help="2: also time the batch as two halves on two streams and report the faster way as `value` (the roofline figures always "
                          "come from the single-stream pass, where launches do not overlap)")
+    ap.add_argument("--skip-three-call", action="store_true",
+                    help="leave the second timed leg (the reference's call sequence per layer) out, e.g. under a profiler")
     ap.add_argument("--unfused", action="store_true", help="run every layer as the reference's three calls (no cross-layer transform fusion)")
     ap.add_argument("--layer-launch", action="store_true", help="experimental: product and both transforms of a layer as one launch (slower)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -590,7 +592,7 @@ def main():
                       "hbm_limited_ceiling_frac": min(1.0, gemm_flops / gemm_bytes * PEAK_HBM_GBS * 1e9 / (PEAK_MFMA_TFLOPS[dtype] * 1e12))},
         "transforms": transforms,
     }
-    if not args.unfused:
+    if not args.unfused and not args.skip_three_call:
         t3 = timed_passes(ctx, lambda: net.forward(fused=False), args.steps, args.warmup)
         result["reference_call_sequence"] = {"value": batch / t3, "unit": "positions/sec", "ms_per_step": 1e3 * t3,
                                              "what": "winograd_input_transform, gemm_batched_v2 and winograd_output_transform as three calls per 3x3 layer, "
