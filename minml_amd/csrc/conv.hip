@@ -16,6 +16,7 @@
 #include "epilogues.hpp"
 #include "gemm_launch.hpp"
 #include "gemm_dma.hpp"
+#include "conv_window.hpp"
 
 #include <cstring>
 
@@ -160,6 +161,24 @@ namespace
 					&& (reinterpret_cast<uintptr_t>(bias) % vbytes == 0);
 			return ep;
 		};
+		if constexpr (sizeof(T) == 2)
+		{
+			/* a narrow 3x3 layer (64 filters in and out) is bound by HBM: every input pixel through LDS once, the weights in registers */
+			const FloatEpilogue<T> ep = make_epilogue();
+			/* the forms that specialise_epilogue fixes at compile time: bias with ReLU or no activation, or the bare product */
+			const bool fixed_form = ep.vectorized && ((ep.bias != nullptr && (ep.act == ACTIVATION_RELU || ep.act == ACTIVATION_LINEAR))
+					|| (ep.bias == nullptr && ep.beta == 0.0f && ep.act == ACTIVATION_LINEAR));
+			if (fast && fixed_form && aligned16(output) && aligned16(add) && conv_window_applies(sizeof(T), filters_in, filters_out, kernel_h, kernel_w, height, width, pixels))
+			{
+				specialise_epilogue(ep, [&](const auto &fixed)
+				{
+					if constexpr (!std::is_same<typename std::decay<decltype(fixed)>::type, FloatEpilogue<T>>::value)
+						launch_conv_window<T>(stream, input, weights, M, height, width, fixed);
+				});
+				MLHIP_CHECK(hipGetLastError());
+				return;
+			}
+		}
 		if (fast && c_bytes % 128 == 0)
 		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */
 			Im2RowDmaRows a_loader;

@@ -157,7 +157,8 @@ namespace mlhip
 					out.v[e] = finish(out.v[e]);
 				return out;
 			}
-			__device__ __forceinline__ void apply(int m, int n, const float (&acc)[4], const Column &col, const Extra &x) const
+			/* the 4 finished results of apply(), for kernels that store them themselves */
+			__device__ __forceinline__ Vec<T, 4> result(const float (&acc)[4], const Column &col, const Extra &x) const
 			{
 				Vec<T, 4> out;
 #pragma unroll
@@ -192,7 +193,11 @@ namespace mlhip
 #pragma unroll
 				for (int e = 0; e < 4; e++)
 					out.v[e] = finish(out.v[e]);
-				out.store(D + static_cast<size_t>(m) * row_stride + n);
+				return out;
+			}
+			__device__ __forceinline__ void apply(int m, int n, const float (&acc)[4], const Column &col, const Extra &x) const
+			{
+				result(acc, col, x).store(D + static_cast<size_t>(m) * row_stride + n);
 			}
 			__device__ __forceinline__ void operator()(int m, int n, const float (&acc)[4]) const
 			{
