@@ -178,6 +178,18 @@ namespace
 				MLHIP_CHECK(hipGetLastError());
 				return;
 			}
+			/* 64 -> 64 filters 5 x 5: the same with the K axis split among the wavefronts */
+			if (fast && fixed_form && aligned16(output) && aligned16(add)
+					&& conv_window_split_applies<ConvSplit5x5x64>(sizeof(T), filters_in, filters_out, kernel_h, kernel_w, height, width, pixels))
+			{
+				specialise_epilogue(ep, [&](const auto &fixed)
+				{
+					if constexpr (!std::is_same<typename std::decay<decltype(fixed)>::type, FloatEpilogue<T>>::value)
+						launch_conv_window_split<T, ConvSplit5x5x64>(stream, input, weights, M, height, width, fixed);
+				});
+				MLHIP_CHECK(hipGetLastError());
+				return;
+			}
 		}
 		if (fast && c_bytes % 128 == 0)
 		{ /* every 128-byte chunk of K lies within one tap: the direct-to-LDS engine */

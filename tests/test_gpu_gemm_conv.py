@@ -287,44 +287,46 @@ def test_convolution_linearity_at_full_size(ctx):
     assert np.array_equal(outs[0][100:101], sample)
 
 
+@pytest.mark.parametrize("channels,k", [(64, 3), (64, 5), (128, 3)])
 @pytest.mark.parametrize("shape", [(1, 19, 19), (2, 7, 5), (3, 30, 9), (64, 19, 19), (5, 1, 40), (2, 3, 100), (1, 2, 130)])
-def test_narrow_3x3_convolution(ctx, shape):
-    """3x3 convolutions with 64 filters in and out in fp16 (the windowed kernel where the image is narrow enough for its pixel ring, the tile
-    engine beyond that) against the oracle's explicit convolution, in every form the epilogue takes: bias + residual + ReLU, bias + ReLU,
-    bias + residual, bias alone, and the bare product. Images of one row, of one column less than the ring allows, and batches whose
-    pixel ranges span several units per workgroup."""
-    rng = np.random.default_rng(sum(shape))
+def test_narrow_convolution(ctx, shape, channels, k):
+    """Convolutions of narrow fp16 layers (64 filters in and out, 3x3 and 5x5, 128 filters 3x3: the windowed kernels where the image is narrow enough for
+    their pixel ring, the tile engine beyond that) against the oracle's explicit convolution, in every form the epilogue takes: bias +
+    residual + ReLU, bias + ReLU, bias + residual, bias alone, and the bare product. Images of one row, of widths on both sides of what the
+    ring allows, and batches whose pixel ranges span several units per workgroup."""
+    rng = np.random.default_rng(sum(shape) + channels + k)
     b, h, w = shape
-    x = random_tensor(rng, (b, h, w, 64), "float16")
-    wt = random_tensor(rng, (64, 3, 3, 64), "float16", (2.0 / (9 * 64)) ** 0.5)
-    bias = random_tensor(rng, (64,), "float16")
-    add = random_tensor(rng, (b, h, w, 64), "float16")
+    x = random_tensor(rng, (b, h, w, channels), "float16")
+    wt = random_tensor(rng, (channels, k, k, channels), "float16", (2.0 / (k * k * channels)) ** 0.5)
+    bias = random_tensor(rng, (channels,), "float16")
+    add = random_tensor(rng, (b, h, w, channels), "float16")
     dx, dw, db, da = (ml.toDevice(ctx, a) for a in (x, wt, bias, add))
     O.set_num_threads(8)
     for with_bias, with_add, act in ((True, True, "relu"), (True, False, "relu"), (True, True, "linear"), (True, False, "linear"), (False, False, "linear")):
-        dy = ml.Tensor((b, h, w, 64), "float16")
+        dy = ml.Tensor((b, h, w, channels), "float16")
         ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, db if with_bias else None, da if with_add else None, act)
         want = O.conv2d_forward(x, wt, bias if with_bias else None, add if with_add else None, O.RELU if act == "relu" else O.LINEAR)
         assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (with_bias, with_add, act)
 
 
-def test_narrow_3x3_convolution_at_full_size(ctx):
-    """Config 4's narrowest 3x3 row at its full size (B = 512, 19x19, 64 channels, fp16, bias + residual + ReLU): positions are independent
-    (a 2-position launch reproduces its slice of the full launch bit for bit), the first, the last and positions between match the oracle."""
-    rng = np.random.default_rng(464)
+@pytest.mark.parametrize("channels,k", [(64, 3), (64, 5), (128, 3)])
+def test_narrow_convolution_at_full_size(ctx, channels, k):
+    """Config 4's narrow rows at their full size (B = 512, 19x19, fp16, bias + residual + ReLU): positions are independent (a 2-position
+    launch reproduces its slice of the full launch bit for bit), the first, the last and positions between match the oracle."""
+    rng = np.random.default_rng(464 + channels + k)
     b = 512
-    x = random_tensor(rng, (b, 19, 19, 64), "float16")
-    wt = random_tensor(rng, (64, 3, 3, 64), "float16", (2.0 / (9 * 64)) ** 0.5)
-    bias = random_tensor(rng, (64,), "float16", 0.01)
-    add = random_tensor(rng, (b, 19, 19, 64), "float16")
+    x = random_tensor(rng, (b, 19, 19, channels), "float16")
+    wt = random_tensor(rng, (channels, k, k, channels), "float16", (2.0 / (k * k * channels)) ** 0.5)
+    bias = random_tensor(rng, (channels,), "float16", 0.01)
+    add = random_tensor(rng, (b, 19, 19, channels), "float16")
     dx, dw, db, da = (ml.toDevice(ctx, a) for a in (x, wt, bias, add))
-    dy = ml.Tensor((b, 19, 19, 64), "float16")
+    dy = ml.Tensor((b, 19, 19, channels), "float16")
     ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, db, da, "relu")
     got = dy.copyToHost(ctx)
-    per = 19 * 19 * 64
+    per = 19 * 19 * channels
     for first in (0, 1, 255, 510):
-        part = ml.Tensor((2, 19, 19, 64), "float16")
-        ml.convolutionImplicitGemmForward(ctx, dx.view((2, 19, 19, 64), first * per), dw, part, db, da.view((2, 19, 19, 64), first * per), "relu")
+        part = ml.Tensor((2, 19, 19, channels), "float16")
+        ml.convolutionImplicitGemmForward(ctx, dx.view((2, 19, 19, channels), first * per), dw, part, db, da.view((2, 19, 19, channels), first * per), "relu")
         assert mismatches(part.copyToHost(ctx), got[first:first + 2]) == 0
     O.set_num_threads(8)
     sample = list(range(0, 512, 37)) + [511]
