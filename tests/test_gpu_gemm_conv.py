@@ -309,6 +309,30 @@ def test_narrow_convolution(ctx, shape, channels, k):
         assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (with_bias, with_add, act)
 
 
+@pytest.mark.parametrize("k", [3, 5])
+def test_narrow_convolution_random_shapes(ctx, k):
+    """The windowed kernels on 40 seeded random tensor shapes (1 to 24 images of 1 to 45 rows and columns): their pixel ranges, ring
+    wrap-arounds, block-aligned and ragged range ends, images smaller than a unit and ranges that span many images all differ from shape
+    to shape. Alternately bias + residual + ReLU and the bare product, against the oracle's explicit convolution."""
+    rng = np.random.default_rng(9000 + k)
+    O.set_num_threads(8)
+    wt = random_tensor(rng, (64, k, k, 64), "float16", (2.0 / (k * k * 64)) ** 0.5)
+    bias = random_tensor(rng, (64,), "float16")
+    dw, db = ml.toDevice(ctx, wt), ml.toDevice(ctx, bias)
+    for case in range(40):
+        b, h, w = int(rng.integers(1, 25)), int(rng.integers(1, 46)), int(rng.integers(1, 46))
+        x = random_tensor(rng, (b, h, w, 64), "float16")
+        add = random_tensor(rng, (b, h, w, 64), "float16")
+        dy = ml.Tensor((b, h, w, 64), "float16")
+        if case % 2 == 0:
+            ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), dw, dy, db, ml.toDevice(ctx, add), "relu")
+            want = O.conv2d_forward(x, wt, bias, add, O.RELU)
+        else:
+            ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), dw, dy, None, None, "linear")
+            want = O.conv2d_forward(x, wt)
+        assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (case, b, h, w)
+
+
 @pytest.mark.parametrize("channels,k", [(64, 3), (64, 5), (128, 3)])
 def test_narrow_convolution_at_full_size(ctx, channels, k):
     """Config 4's narrow rows at their full size (B = 512, 19x19, fp16, bias + residual + ReLU): positions are independent (a 2-position
