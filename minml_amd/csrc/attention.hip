@@ -89,12 +89,17 @@ namespace
 			}
 		}
 	}
-	/* the same with the row held in registers between the two passes: ITEMS vectors of VEC elements per lane, columns <= 64 * VEC * ITEMS */
-	template<typename T, int VEC, int ITEMS>
+	/*
+	 * The same with the row held in registers between the two passes: ITEMS vectors of VEC elements per lane, columns <= 64 * VEC * ITEMS.
+	 * A wavefront takes UNROLL rows at a time and requests all of them before it reduces the first: with one row per wavefront the
+	 * launch is a procession of short-lived wavefronts that each wait out one memory latency (19.5 us for 57 600 rows of 256 halfs,
+	 * 3.0 TB/s).
+	 */
+	template<typename T, int VEC, int ITEMS, int UNROLL>
 	__global__ __launch_bounds__(256) void kernel_rmsnorm_in_registers(T *output, const T *input, const T *weights, size_t rows, int columns)
 	{
 		const int lane = threadIdx.x & 63;
-		const size_t stride = static_cast<size_t>(gridDim.x) * 4;
+		const size_t stride = static_cast<size_t>(gridDim.x) * 4 * UNROLL;
 		const float inv_columns = 1.0f / static_cast<float>(columns);
 		Vec<T, VEC> gamma[ITEMS];
 #pragma unroll
@@ -107,35 +112,45 @@ namespace
 			if (weights != nullptr && j < columns)
 				gamma[i].load(weights + j);
 		}
-		for (size_t row = static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6); row < rows; row += stride)
+		for (size_t first = (static_cast<size_t>(blockIdx.x) * 4 + (threadIdx.x >> 6)) * UNROLL; first < rows; first += stride)
 		{
-			const T *src = input + row * columns;
-			T *dst = output + row * columns;
-			Vec<T, VEC> x[ITEMS];
-			float sum_square = 0.0f;
+			Vec<T, VEC> x[UNROLL][ITEMS];
 #pragma unroll
-			for (int i = 0; i < ITEMS; i++)
+			for (int u = 0; u < UNROLL; u++)
 			{
-				const int j = (lane + 64 * i) * VEC;
-				x[i].zero();
-				if (j < columns)
-					x[i].load(src + j);
+				const T *src = input + (first + u) * columns;
 #pragma unroll
-				for (int e = 0; e < VEC; e++)
-					sum_square = fmaf(x[i].v[e], x[i].v[e], sum_square);
+				for (int i = 0; i < ITEMS; i++)
+				{
+					const int j = (lane + 64 * i) * VEC;
+					x[u][i].zero();
+					if (j < columns && first + u < rows)
+						x[u][i].load(src + j);
+				}
 			}
-			sum_square = wave_sum(sum_square);
-			const float rms = sqrtf(sum_square * inv_columns);
-			const float inv_rms = 1.0f / (1.0e-6f + rms);
 #pragma unroll
-			for (int i = 0; i < ITEMS; i++)
+			for (int u = 0; u < UNROLL; u++)
 			{
-				const int j = (lane + 64 * i) * VEC;
+				float sum_square = 0.0f;
 #pragma unroll
-				for (int e = 0; e < VEC; e++)
-					x[i].v[e] = (gamma[i].v[e] * x[i].v[e]) * inv_rms;
-				if (j < columns)
-					x[i].store(dst + j);
+				for (int i = 0; i < ITEMS; i++)
+#pragma unroll
+					for (int e = 0; e < VEC; e++)
+						sum_square = fmaf(x[u][i].v[e], x[u][i].v[e], sum_square);
+				sum_square = wave_sum(sum_square);
+				const float rms = sqrtf(sum_square * inv_columns);
+				const float inv_rms = 1.0f / (1.0e-6f + rms);
+				T *dst = output + (first + u) * columns;
+#pragma unroll
+				for (int i = 0; i < ITEMS; i++)
+				{
+					const int j = (lane + 64 * i) * VEC;
+#pragma unroll
+					for (int e = 0; e < VEC; e++)
+						x[u][i].v[e] = (gamma[i].v[e] * x[u][i].v[e]) * inv_rms;
+					if (j < columns && first + u < rows)
+						x[u][i].store(dst + j);
+				}
 			}
 		}
 	}
@@ -144,16 +159,19 @@ namespace
 	{
 		constexpr int WIDE = 16 / sizeof(T);
 		const unsigned int groups = static_cast<unsigned int>(std::min<size_t>((rows + 3) / 4, 65536));
+		/* the in-register kernels take 4 rows (2 for the longest rows) per wavefront at a time */
+		const unsigned int groups4 = static_cast<unsigned int>(std::min<size_t>((rows + 15) / 16, 65536));
+		const unsigned int groups2 = static_cast<unsigned int>(std::min<size_t>((rows + 7) / 8, 65536));
 		const bool aligned = (reinterpret_cast<uintptr_t>(input) | reinterpret_cast<uintptr_t>(output) | reinterpret_cast<uintptr_t>(weights)) % 16 == 0;
 		/* rows of up to 64 * WIDE * 4 elements stay in registers; the vector width shrinks for short rows so that all 64 lanes have work */
 		if (aligned && columns % WIDE == 0 && columns > 64 * WIDE / 2 && columns <= 64 * WIDE)
-			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 1>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 1, 4>), dim3(groups4), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else if (aligned && columns % WIDE == 0 && columns > 64 * WIDE && columns <= 64 * WIDE * 2)
-			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 2>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 2, 4>), dim3(groups4), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else if (aligned && columns % WIDE == 0 && columns > 64 * WIDE * 2 && columns <= 64 * WIDE * 4)
-			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 4>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE, 4, 2>), dim3(groups2), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else if (aligned && columns % (WIDE / 2) == 0 && columns <= 64 * WIDE / 2)
-			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE / 2, 1>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
+			hipLaunchKernelGGL((kernel_rmsnorm_in_registers<T, WIDE / 2, 1, 4>), dim3(groups4), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else if (aligned && columns % WIDE == 0)
 			hipLaunchKernelGGL((kernel_rmsnorm_forward<T, WIDE>), dim3(groups), dim3(256), 0, stream, output, input, weights, rows, columns);
 		else
