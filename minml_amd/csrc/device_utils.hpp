@@ -196,6 +196,46 @@ namespace mlhip
 		return q;
 	}
 
+	/*
+	 * Division of a 32-bit number by a divisor that is fixed for a launch: a multiplication, two additions and two shifts (the
+	 * branch-free multiply-and-shift form: q = hi(magic * n), result = (((n - q) >> 1) + q) >> shift) instead of the ~30 instructions
+	 * of a division by a run-time value. Exact for every n < 2^32 and every divisor >= 1.
+	 */
+	struct FastDivisor
+	{
+			uint32_t divisor, magic, shift;
+	};
+	inline FastDivisor make_fast_divisor(uint32_t divisor)
+	{
+		FastDivisor f { divisor, 0u, 0u };
+		if (divisor < 2)
+			return f; /* 1 is handled by the device side */
+		uint32_t log2_floor = 31;
+		while (((divisor >> log2_floor) & 1u) == 0)
+			log2_floor--;
+		if ((divisor & (divisor - 1)) == 0)
+			f.shift = log2_floor - 1; /* a power of two: magic 0 */
+		else
+		{
+			const uint64_t numerator = (static_cast<uint64_t>(1) << log2_floor) << 32;
+			uint32_t proposed = static_cast<uint32_t>(numerator / divisor);
+			const uint64_t rest = numerator % divisor;
+			proposed += proposed;
+			if (rest + rest >= divisor)
+				proposed += 1;
+			f.magic = proposed + 1;
+			f.shift = log2_floor;
+		}
+		return f;
+	}
+	__device__ __forceinline__ uint32_t fast_divide(uint32_t n, const FastDivisor &f, uint32_t &remainder)
+	{
+		const uint32_t q = __umulhi(f.magic, n);
+		const uint32_t quotient = (f.divisor == 1u) ? n : ((((n - q) >> 1) + q) >> f.shift);
+		remainder = n - quotient * f.divisor;
+		return quotient;
+	}
+
 	/* activations of the reference (src/backend/cpu/common_math.hpp:40-55, src/backend/cpu/def_misc_kernels.cpp:52-72) */
 	__device__ __forceinline__ float activate(int act, float x)
 	{
