@@ -17,6 +17,7 @@
 #include "gemm_launch.hpp"
 #include "gemm_dma.hpp"
 #include "conv_window.hpp"
+#include "gemm_dma_window.hpp"
 
 #include <algorithm>
 #include <cstring>
@@ -246,6 +247,16 @@ namespace
 			a_loader.c_bytes = static_cast<int>(c_bytes);
 			a_loader.fill = 0;
 			const DenseDmaRows b_loader { reinterpret_cast<const uint8_t*>(weights), filters_out, static_cast<int>(k_bytes) };
+			if constexpr (sizeof(T) == 2)
+				if (conv_dma_window_applies(c_bytes, filters_out, kernel_h, kernel_w, height, width))
+				{ /* the tiles' rows are consecutive pixels: the window of pixels they share enters LDS once per 128-byte slice of the channels */
+					specialise_epilogue(make_epilogue(), [&](const auto &ep)
+					{
+						launch_conv_dma_window<T>(stream, input, weights, M, filters_out, height, width, kernel_h, static_cast<int>(c_bytes), 0u, ep);
+					});
+					MLHIP_CHECK(hipGetLastError());
+					return;
+				}
 			if constexpr (sizeof(T) == 2) /* the fp16 hot path gets its epilogue's common cases fixed at compile time */
 				specialise_epilogue(make_epilogue(), [&](const auto &ep)
 				{

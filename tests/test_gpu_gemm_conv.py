@@ -358,6 +358,53 @@ def test_narrow_convolution_at_full_size(ctx, channels, k):
     assert max_abs_rel(got[sample], want) <= 1e-2
 
 
+@pytest.mark.parametrize("cin,cout,k", [(64, 128, 3), (128, 128, 5), (192, 192, 3), (64, 384, 5), (128, 576, 3), (64, 128, 5)])
+@pytest.mark.parametrize("shape", [(1, 19, 19), (3, 7, 5), (2, 30, 9), (4, 20, 21), (2, 12, 22), (1, 3, 43), (1, 2, 50), (5, 1, 40), (40, 19, 19)])
+def test_windowed_tile_convolution(ctx, shape, cin, cout, k):
+    """fp16 convolutions whose output width is 128 or a multiple of 192: the tile engine takes its A operand from a window of pixels held
+    in LDS (walked slice by slice over the input channels) where the image is narrow enough for the window, and gathers tap by tap
+    beyond that. Images on both sides of that width for 3x3 and 5x5, of one row, smaller than a tile, ragged last tiles, one to three
+    128-byte slices per pixel; every form of the epilogue including one that is not fixed at compile time, against the oracle."""
+    rng = np.random.default_rng(sum(shape) + cin + cout + k)
+    b, h, w = shape
+    x = random_tensor(rng, (b, h, w, cin), "float16")
+    wt = random_tensor(rng, (cout, k, k, cin), "float16", (2.0 / (k * k * cin)) ** 0.5)
+    bias = random_tensor(rng, (cout,), "float16")
+    add = random_tensor(rng, (b, h, w, cout), "float16")
+    dx, dw, db, da = (ml.toDevice(ctx, a) for a in (x, wt, bias, add))
+    O.set_num_threads(8)
+    forms = ((True, True, "relu"), (True, False, "relu"), (True, True, "linear"), (False, False, "linear"), (True, True, "sigmoid"))
+    for with_bias, with_add, act in forms:
+        dy = ml.Tensor((b, h, w, cout), "float16")
+        ml.convolutionImplicitGemmForward(ctx, dx, dw, dy, db if with_bias else None, da if with_add else None, act)
+        want = O.conv2d_forward(x, wt, bias if with_bias else None, add if with_add else None, ml.act_of(act))
+        assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (with_bias, with_add, act)
+
+
+@pytest.mark.parametrize("cin,cout,k", [(64, 128, 5), (128, 192, 3)])
+def test_windowed_tile_convolution_random_shapes(ctx, cin, cout, k):
+    """The window form of the tile engine on 30 seeded random tensor shapes (1 to 12 images of 1 to 45 rows and columns): tile starts
+    anywhere in an image, windows that begin before the tensor or end past it, images smaller than a tile and wider than the window
+    allows all occur. Alternately bias + residual + ReLU and the bare product, against the oracle's explicit convolution."""
+    rng = np.random.default_rng(9100 + cin + k)
+    O.set_num_threads(8)
+    wt = random_tensor(rng, (cout, k, k, cin), "float16", (2.0 / (k * k * cin)) ** 0.5)
+    bias = random_tensor(rng, (cout,), "float16")
+    dw, db = ml.toDevice(ctx, wt), ml.toDevice(ctx, bias)
+    for case in range(30):
+        b, h, w = int(rng.integers(1, 13)), int(rng.integers(1, 46)), int(rng.integers(1, 46))
+        x = random_tensor(rng, (b, h, w, cin), "float16")
+        add = random_tensor(rng, (b, h, w, cout), "float16")
+        dy = ml.Tensor((b, h, w, cout), "float16")
+        if case % 2 == 0:
+            ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), dw, dy, db, ml.toDevice(ctx, add), "relu")
+            want = O.conv2d_forward(x, wt, bias, add, O.RELU)
+        else:
+            ml.convolutionImplicitGemmForward(ctx, ml.toDevice(ctx, x), dw, dy, None, None, "linear")
+            want = O.conv2d_forward(x, wt)
+        assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (case, b, h, w)
+
+
 @pytest.mark.parametrize("channels,k", [(384, 3), (384, 5), (256, 5), (384, 1)])
 def test_config4_full_size_fp16(ctx, channels, k):
     """Config 4 at its full size (B = 512, 19x19 boards, fp16, bias + residual + ReLU) at the widest channel counts: positions are
