@@ -318,88 +318,169 @@ namespace
 	}
 
 	/*
-	 * The same sum with the search taken out of the wavefronts' critical path. One workgroup serves a range of the tokens of ONE image:
-	 * it first inverts the image's routing table in LDS (inverse[token][expert] = the lowest slot of that expert holding the token, or
-	 * "none"), then every wavefront walks its tokens, reads a token's row of the inverse table from LDS and requests the gates and rows
-	 * of all its slots at once. Same additions in the same order as kernel_scatter_tokens, hence the same bits.
+	 * The same sum with the search taken out of the wavefronts' critical path. One workgroup serves a range of the tokens of ONE image.
+	 * It first inverts the image's routing table for its tokens in LDS (inverse[token][expert] = the lowest slot of that expert holding
+	 * the token, or "none") and compacts every token's row of that table into a list of (row of the expert outputs, gate) in expert
+	 * order; then every wavefront walks its tokens: it reads a token's count and list from LDS into scalar registers and requests all
+	 * of the token's rows at once (up to four per step; the count selects a fully unrolled form). Same additions in the same order as
+	 * kernel_scatter_tokens, hence the same bits.
+	 *
+	 * The kernel is bound by the number of instructions a wavefront issues per token, not by memory: a version that requested all
+	 * `experts` rows of every token (absent ones at an offset outside the buffer, skipped by a select) took as long with every request
+	 * outside the buffer as with the real ones. Hence the compact lists (no work for absent experts), the rows' addresses as scalar
+	 * offsets of a buffer descriptor (no per-lane address arithmetic) and no division in the token loop.
 	 */
 	constexpr int SCATTER_NONE = 0x7fffffff;
+	constexpr int SCATTER_OUTSIDE = 0x40000000; /* offset that lies past the end of the descriptor used here */
 	template<typename T, int VEC>
+	__device__ __forceinline__ Vec<T, VEC> scatter_load_row(__amdgpu_buffer_rsrc_t r, int lane_offset, int row_offset)
+	{
+		Vec<T, VEC> out;
+		if constexpr (VEC == 1 && sizeof(T) == 4)
+			out.v[0] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, lane_offset, row_offset, 0));
+		else if constexpr (VEC == 1)
+			out.v[0] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(__builtin_amdgcn_raw_buffer_load_b16(r, lane_offset, row_offset, 0))));
+		else if constexpr (sizeof(T) == 4)
+		{
+			static_assert(VEC == 4, "rows move 16 bytes per lane");
+			typedef uint32_t words __attribute__((ext_vector_type(4)));
+			const words w = __builtin_amdgcn_raw_buffer_load_b128(r, lane_offset, row_offset, 0);
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+				out.v[i] = __builtin_bit_cast(float, static_cast<uint32_t>(w[i]));
+		}
+		else
+		{
+			static_assert(VEC == 4, "rows move 8 bytes per lane");
+			typedef _Float16 halves __attribute__((ext_vector_type(4)));
+			const halves h = __builtin_bit_cast(halves, __builtin_amdgcn_raw_buffer_load_b64(r, lane_offset, row_offset, 0));
+#pragma unroll
+			for (int i = 0; i < 4; i++)
+				out.v[i] = static_cast<float>(h[i]);
+		}
+		return out;
+	}
+	/* adds N listed contributions to acc: all rows requested before the first is used */
+	template<typename T, int VEC, int N>
+	__device__ __forceinline__ void scatter_add_listed(Vec<T, VEC> &acc, const int *list, __amdgpu_buffer_rsrc_t rows, int lane_offset, int row_bytes)
+	{
+#pragma clang fp contract(off)
+		int row[N];
+		float gate[N];
+		Vec<T, VEC> in[N];
+#pragma unroll
+		for (int i = 0; i < N; i++)
+		{
+			row[i] = __builtin_amdgcn_readfirstlane(list[2 * i]);
+			gate[i] = __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(list[2 * i + 1]));
+		}
+#pragma unroll
+		for (int i = 0; i < N; i++)
+			in[i] = scatter_load_row<T, VEC>(rows, lane_offset, row[i] * row_bytes);
+#pragma unroll
+		for (int i = 0; i < N; i++)
+#pragma unroll
+			for (int v = 0; v < VEC; v++)
+			{
+				const float scaled = gate[i] * in[i].v[v];
+				acc.v[v] = acc.v[v] + scaled;
+			}
+	}
+	/* dynamic LDS of kernel_scatter_tokens_by_image for `per_part` tokens per workgroup: inverse table, lists of (row, gate), counts */
+	inline size_t scatter_by_image_lds_bytes(int per_part, int experts)
+	{
+		return static_cast<size_t>(per_part) * (static_cast<size_t>(experts) * 3 + 1) * sizeof(int);
+	}
+	template<typename T, int VEC, bool WITH_BETA>
 	__global__ __launch_bounds__(256) void kernel_scatter_tokens_by_image(const T *x, const T *indices_and_values, T *y, float beta, int tokens, int channels,
 			int experts, int capacity, int splits)
 	{
 #pragma clang fp contract(off)
-		extern __shared__ int inverse[]; /* [tokens][experts] */
+		extern __shared__ int scatter_lds[];
 		const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 		const size_t b = blockIdx.x / splits;
 		const int part = blockIdx.x % splits;
+		const int per_part = (tokens + splits - 1) / splits;
+		const int first = part * per_part, mine = max(min(tokens, first + per_part) - first, 0); /* this workgroup's tokens: first ... first + mine - 1 */
+		int *inverse = scatter_lds; /* [per_part][experts] */
+		int *lists = inverse + per_part * experts; /* [per_part][experts][2]: row of the image's expert outputs, gate as fp32 bits */
+		int *count = lists + per_part * experts * 2; /* [per_part] */
 		const T *index_plane = indices_and_values + (b * 2 + 0) * experts * capacity;
 		const T *gate_plane = indices_and_values + (b * 2 + 1) * experts * capacity;
-		for (int i = threadIdx.x; i < tokens * experts; i += blockDim.x)
+		for (int i = threadIdx.x; i < mine * experts; i += blockDim.x)
 			inverse[i] = SCATTER_NONE;
 		__syncthreads();
 		for (int i = threadIdx.x; i < experts * capacity; i += blockDim.x)
 		{
 			const int e = i / capacity, k = i - e * capacity;
-			const int token = static_cast<int>(Storage<T>::load(index_plane + i));
-			if (token >= 0 && token < tokens)
-				atomicMin(&inverse[token * experts + e], k);
+			const int token = static_cast<int>(Storage<T>::load(index_plane + i)) - first;
+			if (token >= 0 && token < mine)
+				atomicMin(&inverse[token * experts + e], k); /* of duplicates in a hand-made table the lowest slot counts */
 		}
 		__syncthreads();
-		const int per_part = (tokens + splits - 1) / splits;
-		const int first = part * per_part, last = min(tokens, first + per_part);
-		const int channel_blocks = (channels + 64 * VEC - 1) / (64 * VEC);
-		const int items = max(last - first, 0) * channel_blocks;
-		constexpr int GROUP = 8;
-		for (int item = wave; item < items; item += (blockDim.x >> 6))
+		for (int t = threadIdx.x; t < mine; t += blockDim.x)
 		{
-			const int token = first + item / channel_blocks;
-			const int c = ((item % channel_blocks) * 64 + lane) * VEC;
-			const bool active = c < channels;
-			const size_t global_token = b * tokens + token;
-			Vec<T, VEC> acc;
-			acc.zero();
-			if (beta != 0.0f && active)
+			int n = 0;
+			for (int e = 0; e < experts; e++)
 			{
-				acc.load(y + global_token * channels + c);
-#pragma unroll
-				for (int i = 0; i < VEC; i++)
-					acc.v[i] *= beta;
-			}
-			for (int e0 = 0; e0 < experts; e0 += GROUP)
-			{
-				int found[GROUP];
-				float gate[GROUP];
-				Vec<T, VEC> in[GROUP];
-#pragma unroll
-				for (int i = 0; i < GROUP; i++)
-					found[i] = (e0 + i < experts) ? __builtin_amdgcn_readfirstlane(inverse[token * experts + e0 + i]) : SCATTER_NONE;
-#pragma unroll
-				for (int i = 0; i < GROUP; i++)
+				const int slot = inverse[t * experts + e];
+				if (slot != SCATTER_NONE)
 				{
-					gate[i] = 0.0f;
-					in[i].zero();
-					if (found[i] != SCATTER_NONE)
+					lists[(t * experts + n) * 2 + 0] = slot * experts + e;
+					lists[(t * experts + n) * 2 + 1] = __builtin_bit_cast(int, Storage<T>::load(gate_plane + e * capacity + slot));
+					n++;
+				}
+			}
+			count[t] = n;
+		}
+		__syncthreads();
+		/* the image's expert outputs [capacity][experts][channels] behind a buffer descriptor: a row is a scalar offset, a lane's place in
+		 * it the vector offset, and a lane past the end of the row asks outside the buffer, which returns zeros and moves nothing */
+		const int row_bytes = channels * static_cast<int>(sizeof(T));
+		const __amdgpu_buffer_rsrc_t rows = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(x + b * capacity * experts * channels), 0,
+				capacity * experts * row_bytes, 0x00020000);
+		const int channel_blocks = (channels + 64 * VEC - 1) / (64 * VEC);
+		const int waves = blockDim.x >> 6;
+		for (int t = wave; t < mine; t += waves)
+		{
+			const int n = __builtin_amdgcn_readfirstlane(count[t]);
+			T *y_row = y + (b * tokens + first + t) * channels;
+			for (int block = 0; block < channel_blocks; block++)
+			{
+				const int c = (block * 64 + lane) * VEC;
+				const bool active = c < channels;
+				const int lane_offset = active ? c * static_cast<int>(sizeof(T)) : SCATTER_OUTSIDE;
+				Vec<T, VEC> acc;
+				acc.zero();
+				if constexpr (WITH_BETA)
+				{
+					acc.load(y_row + (active ? c : 0));
+#pragma unroll
+					for (int i = 0; i < VEC; i++)
+						acc.v[i] *= beta;
+				}
+				for (int j = 0; j < n; j += 4)
+				{
+					const int *list = lists + (t * experts + j) * 2;
+					switch (min(n - j, 4))
 					{
-						gate[i] = Storage<T>::load(gate_plane + static_cast<size_t>(e0 + i) * capacity + found[i]);
-						if (active)
-							in[i].load(x + ((b * capacity + found[i]) * experts + e0 + i) * channels + c);
+						case 1:
+							scatter_add_listed<T, VEC, 1>(acc, list, rows, lane_offset, row_bytes);
+							break;
+						case 2:
+							scatter_add_listed<T, VEC, 2>(acc, list, rows, lane_offset, row_bytes);
+							break;
+						case 3:
+							scatter_add_listed<T, VEC, 3>(acc, list, rows, lane_offset, row_bytes);
+							break;
+						default:
+							scatter_add_listed<T, VEC, 4>(acc, list, rows, lane_offset, row_bytes);
+							break;
 					}
 				}
-#pragma unroll
-				for (int i = 0; i < GROUP; i++)
-					if (found[i] != SCATTER_NONE)
-					{
-#pragma unroll
-						for (int v = 0; v < VEC; v++)
-						{
-							const float scaled = gate[i] * in[i].v[v];
-							acc.v[v] = acc.v[v] + scaled;
-						}
-					}
+				if (active)
+					acc.store(y_row + c);
 			}
-			if (active)
-				acc.store(y + global_token * channels + c);
 		}
 	}
 
@@ -577,16 +658,23 @@ extern "C"
 			return;
 		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && indices_and_values.data != nullptr, "scatter_tokens_forward: null tensor");
 		const hipStream_t stream = stream_of(context);
-		/* the by-image form needs the inverted table of one image in LDS and a grid of (images x parts) workgroups */
-		const size_t inverse_bytes = static_cast<size_t>(tokens) * experts * sizeof(int);
+		/* the by-image form needs a grid of (images x parts) workgroups, the tables of a part's tokens in LDS, and the expert outputs of
+		 * one image within reach of a buffer descriptor's 32-bit offsets */
 		const int splits = std::max(1, std::min(8, tokens / 16));
-		const bool by_image = experts > 0 && capacity > 0 && inverse_bytes <= 48 * 1024 && static_cast<size_t>(batch) * splits <= 0x7fffffffu;
+		const size_t lds_bytes = scatter_by_image_lds_bytes((tokens + splits - 1) / splits, experts);
+		const size_t image_bytes = static_cast<size_t>(capacity) * experts * channels * size_of(x.dtype);
+		const bool by_image = experts > 0 && capacity > 0 && lds_bytes <= 48 * 1024 && static_cast<size_t>(batch) * splits <= 0x7fffffffu
+				&& image_bytes < 0x40000000u;
 #define MLHIP_SCATTER(T, VEC) \
 		do { \
 			if (by_image) \
 			{ \
-				hipLaunchKernelGGL((kernel_scatter_tokens_by_image<T, VEC>), dim3(static_cast<unsigned int>(batch) * splits), dim3(256), inverse_bytes, stream, \
-						ptr<const T>(x), ptr<const T>(indices_and_values), ptr<T>(y), beta, tokens, channels, experts, capacity, splits); \
+				if (beta != 0.0f) \
+					hipLaunchKernelGGL((kernel_scatter_tokens_by_image<T, VEC, true>), dim3(static_cast<unsigned int>(batch) * splits), dim3(256), lds_bytes, \
+							stream, ptr<const T>(x), ptr<const T>(indices_and_values), ptr<T>(y), beta, tokens, channels, experts, capacity, splits); \
+				else \
+					hipLaunchKernelGGL((kernel_scatter_tokens_by_image<T, VEC, false>), dim3(static_cast<unsigned int>(batch) * splits), dim3(256), lds_bytes, \
+							stream, ptr<const T>(x), ptr<const T>(indices_and_values), ptr<T>(y), beta, tokens, channels, experts, capacity, splits); \
 				break; \
 			} \
 			const size_t wavefronts = total_tokens * ((channels + 64 * VEC - 1) / (64 * VEC)); \

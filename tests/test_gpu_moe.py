@@ -84,7 +84,11 @@ def test_hash_routing(ctx):
 @pytest.mark.parametrize("dtype", ["float32", "float16"])
 @pytest.mark.parametrize("shape,experts,capacity", [((2, 15, 15, 256), 8, 56), ((2, 5, 7, 12), 3, 40), ((1, 4, 4, 7), 2, 5),
                                                     ((2, 6, 6, 16), 12, 5),      # more experts than one group of eight
-                                                    ((1, 19, 19, 8), 40, 12)])   # inverted table too large for LDS: the scanning form
+                                                    ((1, 19, 19, 8), 40, 12),    # inverted table too large for LDS: the scanning form
+                                                    ((1, 6, 6, 600), 4, 20),     # rows longer than one wavefront's 256 elements, the last piece ragged
+                                                    ((2, 3, 3, 16), 5, 9), ((2, 3, 3, 16), 6, 9), ((2, 3, 3, 16), 7, 9),
+                                                    ((2, 3, 3, 16), 8, 9),       # every expert holds every token: 5 to 8 contributions per token
+                                                    ((1, 3, 3, 5), 11, 9)])      # the same through the one-element form
 def test_gather_and_scatter(ctx, dtype, shape, experts, capacity):
     rng = np.random.default_rng(sum(shape))
     b, h, w, c = shape
