@@ -232,6 +232,43 @@ namespace
 		}
 	}
 
+	/* the same for fewer than 2^32 groups: the flat index is split by multiplications instead of 64-bit divisions, which were most of
+	 * the instructions of a thread that moves 16 bytes; whether the old value takes part is fixed at compile time */
+	template<typename T, int VEC, bool WITH_BETA>
+	__global__ __launch_bounds__(256) void kernel_gather_tokens_fast(const T *x, const T *indices_and_values, T *y, float beta, uint32_t groups, int tokens,
+			int channels, FastDivisor by_pieces, FastDivisor by_experts, FastDivisor by_capacity)
+	{
+		const uint32_t experts = by_experts.divisor, capacity = by_capacity.divisor;
+		for (uint64_t g64 = static_cast<uint64_t>(blockIdx.x) * blockDim.x + threadIdx.x; g64 < groups; g64 += static_cast<uint64_t>(gridDim.x) * blockDim.x)
+		{
+			uint32_t piece, e, k;
+			const uint32_t row = fast_divide(static_cast<uint32_t>(g64), by_pieces, piece); /* (b * K + k) * E + e */
+			const uint32_t bk = fast_divide(row, by_experts, e);
+			const uint32_t b = fast_divide(bk, by_capacity, k);
+			const int c = static_cast<int>(piece) * VEC;
+			const int token = static_cast<int>(Storage<T>::load(indices_and_values + (static_cast<size_t>(b * 2u) * experts + e) * capacity + k));
+			Vec<T, VEC> out;
+			out.zero();
+			T *y_piece = y + static_cast<size_t>(row) * channels + c;
+			if constexpr (WITH_BETA)
+			{
+				out.load(y_piece);
+#pragma unroll
+				for (int i = 0; i < VEC; i++)
+					out.v[i] *= beta;
+			}
+			if (token >= 0)
+			{
+				Vec<T, VEC> in;
+				in.load(x + (static_cast<size_t>(b) * tokens + token) * channels + c);
+#pragma unroll
+				for (int i = 0; i < VEC; i++)
+					out.v[i] = in.v[i] + out.v[i];
+			}
+			out.store(y_piece);
+		}
+	}
+
 	/*
 	 * One wavefront per token and block of 64 * VEC channels: the slots that hold the token are found by scanning the image's index
 	 * table expert by expert (a token occupies at most one slot per expert), and their gated rows are summed in fp32 in that order.
@@ -620,8 +657,24 @@ extern "C"
 			return;
 		MLHIP_REQUIRE(x.data != nullptr && y.data != nullptr && indices_and_values.data != nullptr, "gather_tokens_forward: null tensor");
 		const hipStream_t stream = stream_of(context);
-#define MLHIP_GATHER(T, VEC) hipLaunchKernelGGL((kernel_gather_tokens<T, VEC>), dim3(grid_for(rows * (channels / VEC))), dim3(256), 0, stream, ptr<const T>(x), \
-		ptr<const T>(indices_and_values), ptr<T>(y), beta, rows * (channels / VEC), tokens, channels, experts, capacity)
+#define MLHIP_GATHER(T, VEC) \
+		do { \
+			const size_t groups = rows * (channels / VEC); \
+			if (groups <= 0xffffffffu) \
+			{ \
+				const FastDivisor by_pieces = make_fast_divisor(static_cast<uint32_t>(channels / VEC)), by_experts = make_fast_divisor(static_cast<uint32_t>(experts)), \
+						by_capacity = make_fast_divisor(static_cast<uint32_t>(capacity)); \
+				if (beta != 0.0f) \
+					hipLaunchKernelGGL((kernel_gather_tokens_fast<T, VEC, true>), dim3(grid_for(groups)), dim3(256), 0, stream, ptr<const T>(x), \
+							ptr<const T>(indices_and_values), ptr<T>(y), beta, static_cast<uint32_t>(groups), tokens, channels, by_pieces, by_experts, by_capacity); \
+				else \
+					hipLaunchKernelGGL((kernel_gather_tokens_fast<T, VEC, false>), dim3(grid_for(groups)), dim3(256), 0, stream, ptr<const T>(x), \
+							ptr<const T>(indices_and_values), ptr<T>(y), beta, static_cast<uint32_t>(groups), tokens, channels, by_pieces, by_experts, by_capacity); \
+			} \
+			else \
+				hipLaunchKernelGGL((kernel_gather_tokens<T, VEC>), dim3(grid_for(groups)), dim3(256), 0, stream, ptr<const T>(x), \
+						ptr<const T>(indices_and_values), ptr<T>(y), beta, groups, tokens, channels, experts, capacity); \
+		} while (0)
 		if (x.dtype == DTYPE_FLOAT16)
 		{
 			if (vector_ok<half_t>(channels, 8, x.data, y.data))
