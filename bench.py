@@ -366,6 +366,18 @@ def run_conv_sweep(args, ml):
         rows.append({"channels": chans, "kernel_size": k, "avg_launch_us": t * 1e6, "launches_timed": n, "bound": "hbm" if hbm else "mfma",
                      "achieved": achieved, "peak": peak, "unit": "GB/s" if hbm else "TFLOP/s", "frac": achieved / peak,
                      "algorithmic_bytes": nbytes, "algorithmic_flops": flops})
+    def kernel_of(chans, k):
+        """which kernel conv.hip runs for a layer of the sweep (19x19 boards, fp16, C -> C filters, bias + residual + ReLU)"""
+        if k == 1:
+            return "kernel_gemm_stream_wide_nt<fp16> (1x1: the pixels are the GEMM's rows)"
+        if chans == 64:
+            return "kernel_conv_window<fp16>" if k == 3 else "kernel_conv_window_split<fp16>"
+        if chans % 256 != 0 and (chans % 192 == 0 or chans == 128):
+            return "kernel_conv_dma_window<fp16> (tile engine, A operand from a window of pixels in LDS)"
+        return "kernel_gemm_dma<fp16, im2row> (tile engine, gathered A operand)"
+
+    for r in rows:
+        r["kernel"] = kernel_of(r["channels"], r["kernel_size"])
     slowest = max(rows, key=lambda r: r["avg_launch_us"])
     total_flops = sum(r["algorithmic_flops"] for r in rows)
     result = {
@@ -376,8 +388,8 @@ def run_conv_sweep(args, ml):
                    "epilogue": "bias + residual + ReLU inside the convolution kernel", "step": "the 12 layers one after the other"},
         "tflops_executed": total_flops / t_step / 1e12,
         "roofline": {"bound": slowest["bound"], "achieved": slowest["achieved"], "peak": slowest["peak"], "unit": slowest["unit"], "frac": slowest["frac"],
-                     "traffic": None, "kernel": "kernel_gemm_dma<fp16, im2row, bias + residual + ReLU> (C=%d, k=%d: M=%d N=%d K=%d)"
-                     % (slowest["channels"], slowest["kernel_size"], pix, slowest["channels"], slowest["kernel_size"] ** 2 * slowest["channels"]),
+                     "traffic": None, "kernel": "%s, bias + residual + ReLU (C=%d, k=%d: M=%d N=%d K=%d)"
+                     % (slowest["kernel"], slowest["channels"], slowest["kernel_size"], pix, slowest["channels"], slowest["kernel_size"] ** 2 * slowest["channels"]),
                      "algorithmic_flops": slowest["algorithmic_flops"], "algorithmic_bytes": slowest["algorithmic_bytes"],
                      "launches_timed": slowest["launches_timed"], "avg_launch_us": slowest["avg_launch_us"]},
         "rows": rows,
