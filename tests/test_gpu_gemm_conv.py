@@ -405,7 +405,7 @@ def test_windowed_tile_convolution_random_shapes(ctx, cin, cout, k):
         assert max_abs_rel(dy.copyToHost(ctx), want) <= 1e-2, (case, b, h, w)
 
 
-@pytest.mark.parametrize("channels,k", [(384, 3), (384, 5), (256, 5), (384, 1)])
+@pytest.mark.parametrize("channels,k", [(384, 3), (384, 5), (256, 5), (384, 1), (128, 5), (256, 3)])
 def test_config4_full_size_fp16(ctx, channels, k):
     """Config 4 at its full size (B = 512, 19x19 boards, fp16, bias + residual + ReLU) at the widest channel counts: positions are
     independent (a 2-position launch reproduces its slice of the full launch bit for bit: every output's reduction runs over K in the
